@@ -18,6 +18,7 @@ from __future__ import annotations
 from typing import Any, Dict, Optional, Type
 
 from .base import ConfigError, read_config_json
+from .buketar import BuketarConfig
 from .qwen3 import Qwen3Config
 from .spec import ModelSpec
 
@@ -41,6 +42,8 @@ def resolve_architecture(raw: Dict[str, Any]) -> Type:
     archs = raw.get("architectures") or []
     if isinstance(archs, str):
         archs = [archs]
+    if isinstance(raw.get("architecture"), str):             # (a config.json that names one architecture under the singular key)
+        archs = list(archs) + [raw["architecture"]]
     for a in archs:
         if a in _BY_ARCHITECTURE:
             return _BY_ARCHITECTURE[a]
@@ -66,3 +69,4 @@ def load_spec(model_dir: str) -> ModelSpec:
 
 
 register_architecture(Qwen3Config)
+register_architecture(BuketarConfig)

@@ -38,16 +38,19 @@ class PositionSpec:
     angle = position * theta**(-2i/rot_dim); pairing "half" pairs feature i
     with i + rot_dim/2, "interleaved" pairs 2i with 2i+1.
     kind "none": nothing is applied.
-    `scaling`: None, or a law that changes the angles' frequencies, as (name, factor): ("linear", f)
-    divides every frequency by f (positions are read as position / f).  A law that has no entry in
-    the position part is refused by name when the part is built.
+    `scaling`: None, or a law that changes the angles' frequencies, as (name, factor, ...): ("linear", f)
+    divides every frequency by f (positions are read as position / f); ("yarn", factor, original, fast,
+    slow) divides the frequencies of the pairs that make fewer than `slow` turns over `original` positions
+    by `factor`, keeps those that make more than `fast`, ramps linearly between them, and multiplies cos
+    and sin by 0.1 ln(factor) + 1.  A law that has no entry in the position part is refused by name when
+    the part is built.
     """
     kind: str = "rope"
     head_dim: int = 0
     rot_dim: int = 0
     theta: float = 10000.0
     pairing: str = "half"
-    scaling: Optional[Tuple[str, float]] = None
+    scaling: Optional[Tuple] = None
 
 
 @dataclass(frozen=True)
@@ -82,12 +85,81 @@ class GatedMlpSpec:
 
 
 @dataclass(frozen=True)
+class LatentAttentionSpec:
+    """Softmax attention whose keys and values are products of one low-rank row a token.
+
+    q = W_q h, head by head [head_dim plain | rot_dim rotated]; W_dkv h = [kv_rank latent | rot_dim key part shared
+    by the heads]; the latent is RMS-normed (`norm_eps`); a head's plain key is W_uk c, its value W_uv c
+    (`v_dim` wide); score = (q_plain . k_plain + q_rot . k_rot) * scale.  Only the normed latent and the rotated
+    key part are cached.  `position.rot_dim` of the `rot_dim` rotated features turn.  `gate`: the joined heads are
+    multiplied by sigmoid(W_g h) before the output projection."""
+    hidden: int
+    n_heads: int
+    head_dim: int
+    rot_dim: int
+    v_dim: int
+    kv_rank: int
+    position: PositionSpec
+    scale: float
+    norm_eps: float
+    gate: bool = True
+    window: Optional[int] = None
+    kind: str = "latent_attention"
+
+
+@dataclass(frozen=True)
+class GatedRecurrenceSpec:
+    """The real-gated linear recurrent unit behind a causal convolution a channel, beside a GELU branch:
+    y = gelu_tanh(W_y h + b), u = conv(W_x h + b); r, i = sigmoid of block-diagonal products of u (`blocks` equal
+    parts); a = exp(-decay * r * softplus(lam)); S <- a S + sqrt(1 - a^2) i u; output W_o (S * y)."""
+    hidden: int
+    width: int
+    blocks: int
+    conv: int                      # taps of the convolution; the last meets the current token
+    decay: float = 8.0
+    kind: str = "rglru"
+
+
+@dataclass(frozen=True)
+class RoutedExpertsSpec:
+    """`experts` gated feed-forwards of which a token runs `top`, chosen by the router's scores (`score`:
+    "sigmoid" of each logit, or "softmax" over all); weights = score * `scale`, over the chosen ones
+    renormalised to 1 first with `renormalize`.  An expert: g = min(W_gate h, limit), u = clamp(W_up h, -limit,
+    limit), W_down (g * sigmoid(alpha g) * (u + 1)).  No biases."""
+    hidden: int
+    intermediate: int
+    experts: int
+    top: int
+    scale: float = 1.0
+    limit: float = 7.0
+    alpha: float = 1.702
+    score: str = "sigmoid"
+    renormalize: bool = False
+    kind: str = "routed_experts"
+
+
+@dataclass(frozen=True)
+class StreamsSpec:
+    """How a layer's sub-layers stand around `streams` residual streams (kept in 32-bit): sub-layer q reads
+    sum_s in_q[s] x_s through its norm, its output is scaled feature by feature (`layer_scale`), and the streams
+    become x_t = sum_s mix_q[s, t] x_s + out_q[t] * y.  `connections` False: no such tensors, every coefficient
+    is 1 (with one stream: the ordinary residual sum).  Tensor names: `prefix` + "hc<q>.in" / ".out" / ".mix" and
+    `prefix` + "ls<q>" for q = 1 (mixer) and 2 (feed-forward)."""
+    streams: int
+    hidden: int
+    prefix: str
+    connections: bool = True
+    layer_scale: bool = True
+
+
+@dataclass(frozen=True)
 class LayerSpec:
     """One residual block: which parts, how they are arranged, and the tensor names they load from.
 
     `arrangement` names a registered block class (`parts.register_block`), which says how many
     norms it has and where they stand: "pre_norm" has two, before the mixer and before the
-    feed-forward.  `norms[i]` loads its weight from `norm_names[i]`."""
+    feed-forward; "streams" is pre-norm around several residual streams (`residual`: a `StreamsSpec`) and takes a
+    layer without a feed-forward (`ffn` None, one norm).  `norms[i]` loads its weight from `norm_names[i]`."""
     mixer: Any
     ffn: Any
     norms: Tuple[NormSpec, ...]
@@ -95,6 +167,7 @@ class LayerSpec:
     mixer_prefix: str
     ffn_prefix: str
     arrangement: str = "pre_norm"
+    residual: Any = None
 
 
 @dataclass(frozen=True)
@@ -104,6 +177,17 @@ class EmbeddingSpec:
     hidden: int
     name: str
     kind: str = "embedding"
+
+
+@dataclass(frozen=True)
+class CappedHeadSpec:
+    """A logits head whose logits are capped: cap * tanh(logits / cap) (`cap` None: not capped)."""
+    vocab_size: int
+    hidden: int
+    name: Optional[str]
+    cap: Optional[float] = None
+    required: bool = True
+    kind: str = "capped_lm_head"
 
 
 @dataclass(frozen=True)

@@ -133,6 +133,50 @@ int ia_sample(int* out, const float* logits, void* workspace, int rows, int voca
               const float* temperature, const int* top_k, const float* top_p, const float* min_p,
               const float* u, const int* n_top, float* lp_out, int* lp_ids, hipStream_t stream);
 
+// ---- several residual streams a token (streams.hip) ------------------------------------------------------------
+// streams: 32-bit [n, S, W].  One call adds a sub-layer's output into the streams (x_t <- sum_s mix[s][t] x_s +
+// out[t] * scale * y; y null: skipped; y may be K rows a token with 32-bit weights yw) and forms the next
+// sub-layer's input h = rmsnorm(sum_s in[s] x_s) * w (h null: skipped; rows: only these rows, for a call without y).
+int ia_streams_step(float* streams, const void* y, const float* yw, int K, const float* scale,
+                    const float* mix, const float* outc, const float* inc, const float* w, float eps,
+                    void* h, const int* rows, int n, int S, int W, int y_dtype, int h_dtype, hipStream_t stream);
+int ia_streams_open(float* streams, const void* x, int n, int S, int W, int dtype, hipStream_t stream);
+int ia_softcap(float* x, long long n, float cap, hipStream_t stream);
+
+// ---- latent attention (latent.hip) -------------------------------------------------------------------------------
+int ia_latent_prep(void* q_out, void* k_cache, void* v_cache, const void* proj, const float* norm_w,
+                   const float* cos_t, const float* sin_t, const int* slots, int n, int H, int d, int r,
+                   int rank, int rd, int q_off, int down_off, int ld_proj, int page_size, float eps,
+                   float mag, int dtype, hipStream_t stream);
+// out[t][h][j] = sum_i w[h][j][i] x[t][h][i], optionally times sigmoid(gate[t][h][j])
+int ia_head_product(void* out, const void* x, const void* w, const void* gate, int n, int H, int n_out,
+                    int k_in, long long x_ld, int x_off, int x_head, long long o_ld, int o_off, int o_head,
+                    long long g_ld, int g_off, int x_dtype, int w_dtype, int out_dtype, hipStream_t stream);
+
+// ---- gated linear recurrence behind a short convolution (recurrence.hip) ----------------------------------------
+int ia_conv_step(float* u, const void* x, const void* taps, const void* bias, const float* state,
+                 const int* token_seq, const int* cu_tokens, const int* state_slots, int n, int width, int k,
+                 long long x_ld, int x_off, int dtype, hipStream_t stream);
+int ia_rglru_scan(void* out, float* state, const float* u, const float* z, const void* bias_r,
+                  const void* bias_i, const void* lam, const void* branch, const void* x,
+                  const int* cu_tokens, const int* state_slots, int n_seqs, int width, int bw, int k,
+                  float decay, long long b_ld, int b_off, long long x_ld, int x_off, int dtype,
+                  hipStream_t stream);
+
+// ---- routed experts (experts.hip) --------------------------------------------------------------------------------
+// score_fn: 0 sigmoid, 1 softmax over all experts
+int ia_route(int* sel, float* weight, const void* h, const float* router, int n, int W, int E, int top,
+             float scale, int score_fn, int renorm, int dtype, hipStream_t stream);
+int ia_route_tiles(int pairs, int E);
+int ia_route_plan(int* order, int* tile_expert, int* tile_first, int* tile_rows, int* meta, const int* sel,
+                  int pairs, int E, hipStream_t stream);
+int ia_experts_gate_up(void* act, const void* h, const void* w_gu, const int* order, const int* tile_expert,
+                       const int* tile_first, const int* tile_rows, const int* meta, int pairs, int E, int top,
+                       int W, int ff, float limit, float alpha, int dtype, hipStream_t stream);
+int ia_experts_down(float* y, const void* act, const void* w_down, const int* order, const int* tile_expert,
+                    const int* tile_first, const int* tile_rows, const int* meta, int pairs, int E, int W,
+                    int ff, int dtype, hipStream_t stream);
+
 // Built per head size (-DIA_HEAD_DIM) into a library of its own.
 int ia_attention_mfma_head_dim(void);
 long long ia_attention_mfma_workspace(int n, int nq, int splits);

@@ -1,0 +1,231 @@
+// Routed experts: a router scores every expert for a token, the `top` best are run and their outputs added up
+// with the scores as weights.
+//
+//   route      a wave a token: router logits in 32-bit, scores = sigmoid (or softmax), the top experts by score
+//              (ties: the lower index), weights = score * scale (optionally renormalised over the chosen).
+//   plan       one block: the (token, k) pairs ordered by expert, and a table of row tiles (expert, first pair, rows),
+//              all on the device: the host never learns how many tokens an expert got.
+//   gate_up    tile by tile: rows gathered by pair, act(gate, up) in the epilogue.
+//   down       tile by tile: one 32-bit output row a pair; whoever adds the experts up takes the pairs of a token
+//              in the order of k, so a token's sum does not depend on what else is in the batch.
+#include "api.h"
+#include "common.h"
+#include "tile_fma.h"
+
+#define IA_MAX_EXPERTS 256
+#define IA_MAX_TOP 16
+
+enum { IA_SCORE_SIGMOID = 0, IA_SCORE_SOFTMAX = 1 };
+
+template <typename T>
+__global__ __launch_bounds__(64) void route_kernel(int* __restrict__ sel, float* __restrict__ weight,
+                                                   const T* __restrict__ h, const float* __restrict__ wr, int n, int W,
+                                                   int E, int top, float scale, int score_fn, int renorm) {
+    const int t = blockIdx.x, lane = threadIdx.x;
+    const T* row = h + (long long)t * W;
+    float z[IA_MAX_EXPERTS / IA_WAVE];             // expert e lives in lane e % 64, register e / 64
+#pragma unroll
+    for (int q = 0; q < IA_MAX_EXPERTS / IA_WAVE; ++q) z[q] = -INFINITY;
+    for (int e = 0; e < E; ++e) {
+        const float* w = wr + (long long)e * W;
+        float acc = 0.f;
+        for (int c = lane; c < W; c += IA_WAVE) acc = fmaf(ld(row + c), w[c], acc);
+        acc = wave_sum(acc);
+#pragma unroll
+        for (int q = 0; q < IA_MAX_EXPERTS / IA_WAVE; ++q)
+            if (e == q * IA_WAVE + lane) z[q] = acc;
+    }
+    float zmax = -INFINITY, denom = 1.f;
+    if (score_fn == IA_SCORE_SOFTMAX) {
+#pragma unroll
+        for (int q = 0; q < IA_MAX_EXPERTS / IA_WAVE; ++q) zmax = fmaxf(zmax, z[q]);
+        zmax = wave_max(zmax);
+        float s = 0.f;
+#pragma unroll
+        for (int q = 0; q < IA_MAX_EXPERTS / IA_WAVE; ++q) s += z[q] > -INFINITY ? expf(z[q] - zmax) : 0.f;
+        denom = wave_sum(s);
+    }
+    float total = 0.f, mine = 0.f;
+    int mine_e = 0;
+    for (int k = 0; k < top; ++k) {
+        // every lane's best, then the wave's: the largest logit, of equal ones the lower index
+        float best = -INFINITY;
+        int best_e = 0x7fffffff;
+#pragma unroll
+        for (int q = 0; q < IA_MAX_EXPERTS / IA_WAVE; ++q)
+            if (z[q] > best) { best = z[q]; best_e = q * IA_WAVE + lane; }
+#pragma unroll
+        for (int o = IA_WAVE / 2; o > 0; o >>= 1) {
+            const float ob = __shfl_xor(best, o, IA_WAVE);
+            const int oe = __shfl_xor(best_e, o, IA_WAVE);
+            if (ob > best || (ob == best && oe < best_e)) { best = ob; best_e = oe; }
+        }
+#pragma unroll
+        for (int q = 0; q < IA_MAX_EXPERTS / IA_WAVE; ++q)
+            if (best_e == q * IA_WAVE + lane) z[q] = -INFINITY;
+        const float s = score_fn == IA_SCORE_SOFTMAX ? expf(best - zmax) / denom : 1.0f / (1.0f + expf(-best));
+        total += s;
+        if (lane == k) { mine = s; mine_e = best_e; }
+    }
+    if (lane < top) {
+        sel[(long long)t * top + lane] = mine_e;
+        weight[(long long)t * top + lane] = (renorm ? mine / total : mine) * scale;
+    }
+}
+
+// One block.  `order` [pairs]: the pairs grouped by expert; tiles: expert, first place in `order`, rows; meta[0]: tiles.
+__global__ __launch_bounds__(1024) void route_plan_kernel(int* __restrict__ order, int* __restrict__ tile_expert,
+                                                          int* __restrict__ tile_first, int* __restrict__ tile_rows,
+                                                          int* __restrict__ meta, const int* __restrict__ sel, int pairs,
+                                                          int E) {
+    __shared__ int count[IA_MAX_EXPERTS], first[IA_MAX_EXPERTS], tile0[IA_MAX_EXPERTS], cursor[IA_MAX_EXPERTS];
+    for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = cursor[e] = 0;
+    __syncthreads();
+    for (int p = threadIdx.x; p < pairs; p += blockDim.x) atomicAdd(&count[sel[p]], 1);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int at = 0, tiles = 0;
+        for (int e = 0; e < E; ++e) {
+            first[e] = at;
+            tile0[e] = tiles;
+            at += count[e];
+            tiles += (count[e] + IA_TM - 1) / IA_TM;
+        }
+        meta[0] = tiles;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += blockDim.x) {
+        const int tiles = (count[e] + IA_TM - 1) / IA_TM;
+        for (int i = 0; i < tiles; ++i) {
+            tile_expert[tile0[e] + i] = e;
+            tile_first[tile0[e] + i] = first[e] + i * IA_TM;
+            tile_rows[tile0[e] + i] = min(IA_TM, count[e] - i * IA_TM);
+        }
+    }
+    for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
+        const int e = sel[p];
+        order[first[e] + atomicAdd(&cursor[e], 1)] = p;
+    }
+}
+
+// act[place][j] = g' * sigmoid(alpha g') * (u' + 1), g' = min(gate_j . x, limit), u' = clamp(up_j . x, -limit, limit);
+// x = h[pair / top].  w_gu [E][2 ff][W]: an expert's gate rows, then its up rows.
+template <typename T>
+__global__ __launch_bounds__(256) void experts_gate_up_kernel(T* __restrict__ act, const T* __restrict__ h,
+                                                              const T* __restrict__ w_gu, const int* __restrict__ order,
+                                                              const int* __restrict__ tile_expert,
+                                                              const int* __restrict__ tile_first,
+                                                              const int* __restrict__ tile_rows,
+                                                              const int* __restrict__ meta, int top, int W, int ff,
+                                                              float limit, float alpha) {
+    __shared__ TileShared sh;
+    const int tile = blockIdx.y;
+    if (tile >= meta[0]) return;
+    const int e = tile_expert[tile], first = tile_first[tile], rows = tile_rows[tile], col0 = blockIdx.x * IA_TN;
+    float g[2][4], u[2][4];
+    auto xrow = [&](int i) -> const T* { return i < rows ? h + (long long)(order[first + i] / top) * W : nullptr; };
+    const T* wg = w_gu + ((long long)e * 2 * ff + col0) * W;
+    tile_product<T, T, true>(g, u, sh, xrow, wg, wg + (long long)ff * W, ff - col0, W, W);
+    const int ty = threadIdx.x >> 4, tx = threadIdx.x & 15;
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+        const int i = 2 * ty + a;
+        if (i >= rows) continue;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int j = col0 + 4 * tx + b;
+            if (j >= ff) continue;
+            const float gv = fminf(g[a][b], limit), uv = fminf(fmaxf(u[a][b], -limit), limit);
+            st(act + (long long)(first + i) * ff + j, gv / (1.0f + expf(-alpha * gv)) * (uv + 1.0f));
+        }
+    }
+}
+
+// y[pair][c] = down_c . act[place]   (32-bit rows, one a pair)
+template <typename T>
+__global__ __launch_bounds__(256) void experts_down_kernel(float* __restrict__ y, const T* __restrict__ act,
+                                                           const T* __restrict__ w_down, const int* __restrict__ order,
+                                                           const int* __restrict__ tile_expert,
+                                                           const int* __restrict__ tile_first,
+                                                           const int* __restrict__ tile_rows,
+                                                           const int* __restrict__ meta, int W, int ff) {
+    __shared__ TileShared sh;
+    const int tile = blockIdx.y;
+    if (tile >= meta[0]) return;
+    const int e = tile_expert[tile], first = tile_first[tile], rows = tile_rows[tile], col0 = blockIdx.x * IA_TN;
+    float acc[2][4], unused[2][4];
+    auto xrow = [&](int i) -> const T* { return i < rows ? act + (long long)(first + i) * ff : nullptr; };
+    const T* wd = w_down + ((long long)e * W + col0) * ff;
+    tile_product<T, T, false>(acc, unused, sh, xrow, wd, wd, W - col0, ff, ff);
+    const int ty = threadIdx.x >> 4, tx = threadIdx.x & 15;
+#pragma unroll
+    for (int a = 0; a < 2; ++a) {
+        const int i = 2 * ty + a;
+        if (i >= rows) continue;
+        const long long pair = order[first + i];
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            const int c = col0 + 4 * tx + b;
+            if (c < W) y[pair * W + c] = acc[a][b];
+        }
+    }
+}
+
+extern "C" int ia_route(int* sel, float* weight, const void* h, const float* router, int n, int W, int E, int top,
+                        float scale, int score_fn, int renorm, int dtype, hipStream_t stream) {
+    IA_CHECK(n >= 0 && W > 0 && E >= 1 && E <= IA_MAX_EXPERTS && top >= 1 && top <= E && top <= IA_MAX_TOP,
+             "route: n=%d width=%d experts=%d (up to %d) top=%d (up to %d)", n, W, E, IA_MAX_EXPERTS, top, IA_MAX_TOP);
+    IA_CHECK(score_fn == IA_SCORE_SIGMOID || score_fn == IA_SCORE_SOFTMAX, "route: unknown score function %d", score_fn);
+    if (n == 0) return 0;
+    if (dtype == IA_F32)
+        route_kernel<float><<<n, 64, 0, stream>>>(sel, weight, (const float*)h, router, n, W, E, top, scale, score_fn, renorm);
+    else
+        route_kernel<bf16_t><<<n, 64, 0, stream>>>(sel, weight, (const bf16_t*)h, router, n, W, E, top, scale, score_fn, renorm);
+    IA_LAUNCH_CHECK("route");
+    return 0;
+}
+
+// The most tiles that `pairs` pairs over E experts can make: the grids of the two products.
+extern "C" int ia_route_tiles(int pairs, int E) { return (pairs + IA_TM - 1) / IA_TM + (E < pairs ? E : pairs); }
+
+extern "C" int ia_route_plan(int* order, int* tile_expert, int* tile_first, int* tile_rows, int* meta, const int* sel,
+                             int pairs, int E, hipStream_t stream) {
+    IA_CHECK(pairs >= 0 && E >= 1 && E <= IA_MAX_EXPERTS, "route_plan: pairs=%d experts=%d", pairs, E);
+    route_plan_kernel<<<1, 1024, 0, stream>>>(order, tile_expert, tile_first, tile_rows, meta, sel, pairs, E);
+    IA_LAUNCH_CHECK("route_plan");
+    return 0;
+}
+
+extern "C" int ia_experts_gate_up(void* act, const void* h, const void* w_gu, const int* order, const int* tile_expert,
+                                  const int* tile_first, const int* tile_rows, const int* meta, int pairs, int E, int top,
+                                  int W, int ff, float limit, float alpha, int dtype, hipStream_t stream) {
+    IA_CHECK(pairs >= 0 && W > 0 && ff > 0 && top >= 1 && limit > 0.f, "experts_gate_up: bad sizes");
+    if (pairs == 0) return 0;
+    const dim3 grid((ff + IA_TN - 1) / IA_TN, ia_route_tiles(pairs, E));
+    IA_CHECK(grid.y <= 65535, "experts_gate_up: %u row tiles are more than a grid takes", grid.y);
+    if (dtype == IA_F32)
+        experts_gate_up_kernel<float><<<grid, 256, 0, stream>>>((float*)act, (const float*)h, (const float*)w_gu, order,
+                                                                tile_expert, tile_first, tile_rows, meta, top, W, ff, limit, alpha);
+    else
+        experts_gate_up_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)act, (const bf16_t*)h, (const bf16_t*)w_gu, order,
+                                                                 tile_expert, tile_first, tile_rows, meta, top, W, ff, limit, alpha);
+    IA_LAUNCH_CHECK("experts_gate_up");
+    return 0;
+}
+
+extern "C" int ia_experts_down(float* y, const void* act, const void* w_down, const int* order, const int* tile_expert,
+                               const int* tile_first, const int* tile_rows, const int* meta, int pairs, int E, int W,
+                               int ff, int dtype, hipStream_t stream) {
+    IA_CHECK(pairs >= 0 && W > 0 && ff > 0, "experts_down: bad sizes");
+    if (pairs == 0) return 0;
+    const dim3 grid((W + IA_TN - 1) / IA_TN, ia_route_tiles(pairs, E));
+    IA_CHECK(grid.y <= 65535, "experts_down: %u row tiles are more than a grid takes", grid.y);
+    if (dtype == IA_F32)
+        experts_down_kernel<float><<<grid, 256, 0, stream>>>(y, (const float*)act, (const float*)w_down, order, tile_expert,
+                                                             tile_first, tile_rows, meta, W, ff);
+    else
+        experts_down_kernel<bf16_t><<<grid, 256, 0, stream>>>(y, (const bf16_t*)act, (const bf16_t*)w_down, order, tile_expert,
+                                                              tile_first, tile_rows, meta, W, ff);
+    IA_LAUNCH_CHECK("experts_down");
+    return 0;
+}

@@ -1,0 +1,120 @@
+// A gated linear recurrence a channel (the real-gated linear recurrent unit) behind a short causal convolution:
+//     u_t = bias + sum_j taps[j] * in_(t - (k - 1 - j))                       (zeros before a sequence's start)
+//     r_t = sigmoid(zr_t + br),  i_t = sigmoid(zi_t + bi)                    (zr, zi: block-diagonal products of u)
+//     a_t = exp(-c * r_t * softplus(lam)),   S_t = a_t S_(t-1) + sqrt(1 - a_t^2) * i_t * u_t
+//     out_t = S_t * gelu_tanh(branch_t)
+// Gates, decays and the state are 32-bit.  What a request carries from step to step lies in its row of `state`,
+// [slots][k][width] of 32-bit floats: row 0 the recurrent state S, rows 1..k-1 the last k - 1 inputs of the
+// convolution, oldest first.  A new request's row is zero.
+#include "api.h"
+#include "common.h"
+
+// u [n, width] (32-bit) of the step's tokens; reads the inputs that precede a request's portion from its state row.
+template <typename T>
+__global__ void conv_step_kernel(float* __restrict__ u, const T* __restrict__ x, const T* __restrict__ taps,
+                                 const T* __restrict__ bias, const float* __restrict__ state,
+                                 const int* __restrict__ token_seq, const int* __restrict__ cu_tokens,
+                                 const int* __restrict__ state_slots, int width, int k, long long x_ld, int x_off,
+                                 long long total) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int t = (int)(i / width), c = (int)(i - (long long)t * width);
+    const int seq = token_seq[t];
+    const int first = cu_tokens[seq];
+    const float* tail = state + ((long long)state_slots[seq] * k + 1) * width + c;      // rows 1..k-1
+    float acc = bias != nullptr ? ld(bias + c) : 0.f;
+    for (int j = 0; j < k; ++j) {
+        const int src = t - (k - 1 - j);                    // the token this tap meets
+        float v;
+        if (src >= first) v = ld(x + (long long)src * x_ld + x_off + c);
+        else v = tail[(long long)((k - 1) + (src - first)) * width];
+        acc = fmaf(ld(taps + (long long)c * k + j), v, acc);
+    }
+    u[i] = acc;
+}
+
+// One thread a (request, channel) walks the request's tokens in order.  z [n, 2 * width] holds, block by block,
+// [zr of the block | zi of the block] (blocks of `bw` channels).  Afterwards the thread moves the convolution's last
+// inputs into the state row.
+template <typename T>
+__global__ void rglru_scan_kernel(T* __restrict__ out, float* __restrict__ state, const float* __restrict__ u,
+                                  const float* __restrict__ z, const T* __restrict__ bias_r, const T* __restrict__ bias_i,
+                                  const T* __restrict__ lam, const T* __restrict__ branch, const T* __restrict__ x,
+                                  const int* __restrict__ cu_tokens, const int* __restrict__ state_slots, int width,
+                                  int bw, int k, float decay, long long b_ld, int b_off, long long x_ld, int x_off) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= width) return;
+    const int seq = blockIdx.y;
+    const int first = cu_tokens[seq], last = cu_tokens[seq + 1];
+    float* row = state + (long long)state_slots[seq] * k * width + c;
+    const int blk = c / bw, j = c - blk * bw;
+    const long long zr_at = (long long)blk * 2 * bw + j, zi_at = zr_at + bw;
+    const float br = ld(bias_r + c), bi = ld(bias_i + c);
+    const float l = ld(lam + c);
+    const float sp = fmaxf(l, 0.f) + log1pf(expf(-fabsf(l)));             // softplus
+    float S = row[0];
+    for (int t = first; t < last; ++t) {
+        const float r = 1.0f / (1.0f + expf(-(z[(long long)t * 2 * width + zr_at] + br)));
+        const float g = 1.0f / (1.0f + expf(-(z[(long long)t * 2 * width + zi_at] + bi)));
+        const float log_a = -decay * r * sp;
+        const float a = expf(log_a);
+        const float m = sqrtf(-expm1f(2.0f * log_a));                        // sqrt(1 - a^2)
+        S = fmaf(a, S, m * g * u[(long long)t * width + c]);
+        const float bv = ld(branch + (long long)t * b_ld + b_off + c);
+        const float y = 0.5f * bv * (1.0f + tanhf(0.7978845608028654f * (bv + 0.044715f * bv * bv * bv)));
+        st(out + (long long)t * width + c, S * y);
+    }
+    row[0] = S;
+    // the last k - 1 inputs, oldest first: those of this portion, and before them what the row held
+    const int q = last - first;
+    for (int m = 0; m < k - 1; ++m) {
+        const int src = last - (k - 1) + m;
+        float v;
+        if (src >= first) v = ld(x + (long long)src * x_ld + x_off + c);
+        else v = row[(long long)(1 + m + q) * width];                       // (m + q < k - 1 here; read before it is written)
+        row[(long long)(1 + m) * width] = v;
+    }
+}
+
+extern "C" int ia_conv_step(float* u, const void* x, const void* taps, const void* bias, const float* state,
+                            const int* token_seq, const int* cu_tokens, const int* state_slots, int n, int width, int k,
+                            long long x_ld, int x_off, int dtype, hipStream_t stream) {
+    IA_CHECK(n >= 0 && width > 0 && k >= 1 && x_off >= 0 && x_off + width <= x_ld, "conv_step: bad sizes n=%d width=%d taps=%d",
+             n, width, k);
+    const long long total = (long long)n * width;
+    if (total == 0) return 0;
+    const int blocks = (int)((total + 255) / 256);
+    if (dtype == IA_F32)
+        conv_step_kernel<float><<<blocks, 256, 0, stream>>>(u, (const float*)x, (const float*)taps, (const float*)bias, state,
+                                                            token_seq, cu_tokens, state_slots, width, k, x_ld, x_off, total);
+    else
+        conv_step_kernel<bf16_t><<<blocks, 256, 0, stream>>>(u, (const bf16_t*)x, (const bf16_t*)taps, (const bf16_t*)bias,
+                                                             state, token_seq, cu_tokens, state_slots, width, k, x_ld, x_off,
+                                                             total);
+    IA_LAUNCH_CHECK("conv_step");
+    return 0;
+}
+
+extern "C" int ia_rglru_scan(void* out, float* state, const float* u, const float* z, const void* bias_r,
+                             const void* bias_i, const void* lam, const void* branch, const void* x,
+                             const int* cu_tokens, const int* state_slots, int n_seqs, int width, int bw, int k,
+                             float decay, long long b_ld, int b_off, long long x_ld, int x_off, int dtype,
+                             hipStream_t stream) {
+    IA_CHECK(n_seqs >= 0 && width > 0 && bw > 0 && width % bw == 0 && k >= 1, "rglru_scan: bad sizes seqs=%d width=%d block=%d taps=%d",
+             n_seqs, width, bw, k);
+    IA_CHECK(b_off >= 0 && b_off + width <= b_ld && x_off >= 0 && x_off + width <= x_ld, "rglru_scan: the branches do not fit their rows");
+    IA_CHECK(n_seqs <= 65535, "rglru_scan: %d requests are more than a grid takes", n_seqs);
+    if (n_seqs == 0) return 0;
+    const dim3 grid((width + 63) / 64, n_seqs);
+    if (dtype == IA_F32)
+        rglru_scan_kernel<float><<<grid, 64, 0, stream>>>((float*)out, state, u, z, (const float*)bias_r, (const float*)bias_i,
+                                                          (const float*)lam, (const float*)branch, (const float*)x, cu_tokens,
+                                                          state_slots, width, bw, k, decay, b_ld, b_off, x_ld, x_off);
+    else
+        rglru_scan_kernel<bf16_t><<<grid, 64, 0, stream>>>((bf16_t*)out, state, u, z, (const bf16_t*)bias_r,
+                                                           (const bf16_t*)bias_i, (const bf16_t*)lam, (const bf16_t*)branch,
+                                                           (const bf16_t*)x, cu_tokens, state_slots, width, bw, k, decay, b_ld,
+                                                           b_off, x_ld, x_off);
+    IA_LAUNCH_CHECK("rglru_scan");
+    return 0;
+}

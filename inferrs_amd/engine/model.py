@@ -88,6 +88,9 @@ class DecoderModel:
         """Runs the step's tokens through every stop of the schedule (which appends to the
         caches) and returns float32 logits `[n_want, vocab]`."""
         x = self.embedding.forward(ctx)
+        first = self.blocks[self.spec.schedule[0].layer]
+        if hasattr(first, "enter"):                  # an arrangement whose stream is not the embedding's rows
+            x = first.enter(ctx, x)
         pending = None                               # a block's output that is not added to x yet
         for stop, e in enumerate(self.spec.schedule):
             cache = storage.layers.get(self.spec.cache_stop(stop))
@@ -99,6 +102,9 @@ class DecoderModel:
         n_want = ctx.want_rows.numel()
         if n_want == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)
+        last = self.blocks[self.spec.schedule[-1].layer]
+        if hasattr(last, "leave"):                   # such an arrangement hands over the final norm's output itself
+            return self.head.forward(last.leave(ctx, x, pending, ctx.want_rows, self.final_norm))
         if isinstance(pending, ops.Partials):        # the last product is still split along k
             pending = pending.materialize()
         xs = ops.gather_rows(x, ctx.want_rows)

@@ -1179,3 +1179,8 @@ def gated_linear(x, w_gate_up: torch.Tensor, activation: str = "silu",
 def gated_silu_linear(x, w_gate_up: torch.Tensor) -> torch.Tensor:
     """`gated_linear` with SiLU and no bias."""
     return gated_linear(x, w_gate_up, "silu")
+
+
+# ---- several residual streams, latent attention, gated recurrence, routed experts -----------------
+from .mix import (conv_step, experts_forward, head_product, latent_prep, rglru_scan, route, softcap,   # noqa: E402
+                  streams_open, streams_step)

@@ -1,0 +1,233 @@
+"""Python face of the kernels for several residual streams, latent attention, the gated linear
+recurrence and routed experts (`csrc/streams.hip`, `latent.hip`, `recurrence.hip`, `experts.hip`).
+Shape checks on the host, then one C call a kernel; no other implementation stands behind them."""
+from __future__ import annotations
+
+import ctypes
+from typing import Optional, Tuple
+
+import torch
+
+from . import KernelError, _DT, _check, _dev, _dt, _f32, _i32, _p, _stream, library
+
+MAX_STREAMS = 8
+MAX_EXPERTS = 256
+MAX_TOP = 16
+ROW_TILE = 32                 # rows of a tile of the grouped products
+SCORE_FUNCTIONS = {"sigmoid": 0, "softmax": 1}
+
+
+# ---- residual streams -----------------------------------------------------------------------
+
+def streams_open(x: torch.Tensor, n_streams: int) -> torch.Tensor:
+    """Rows [n, width] -> 32-bit streams [n, S, width], every stream a copy of the row."""
+    _dev(x)
+    n, width = x.shape
+    out = torch.empty((n, n_streams, width), dtype=torch.float32, device=x.device)
+    _check(library().ia_streams_open(_p(out), _p(x), n, n_streams, width, _dt(x), _stream()))
+    return out
+
+
+def streams_step(streams: torch.Tensor, *, y: Optional[torch.Tensor] = None, y_weights: Optional[torch.Tensor] = None,
+                 scale: Optional[torch.Tensor] = None, mix: Optional[torch.Tensor] = None,
+                 out: Optional[torch.Tensor] = None, read: Optional[torch.Tensor] = None,
+                 norm_weight: Optional[torch.Tensor] = None, eps: float = 0.0,
+                 h_dtype: Optional[torch.dtype] = None, rows: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
+    """What stands between two sub-layers of a model with S residual streams.
+
+    `y` [n, width] (or [n, K, width] with `y_weights` [n, K], added up in the order of K): the streams become
+    x_t = sum_s mix[s, t] x_s + out[t] * scale * y, in place.  `h_dtype`: returns rmsnorm(sum_s read[s] x_s) *
+    norm_weight in that precision (`read` None: every stream counts once; `rows`: only these rows, for a call
+    without `y`)."""
+    _dev(streams, y, y_weights, scale, mix, out, read, norm_weight, rows)
+    for t, name in ((streams, "streams"), (y_weights, "y_weights"), (scale, "scale"), (mix, "mix"), (out, "out"),
+                    (read, "read"), (norm_weight, "norm weight")):
+        _f32(t, name)
+    n, S, W = streams.shape
+    K = 1
+    if y is not None:
+        if y_weights is not None:
+            K = y_weights.shape[1]
+            if tuple(y.shape) != (n, K, W) or tuple(y_weights.shape) != (n, K):
+                raise KernelError(f"streams_step: y {tuple(y.shape)} and its weights {tuple(y_weights.shape)} do not fit [{n}, K, {W}]")
+        elif tuple(y.shape) != (n, W):
+            raise KernelError(f"streams_step: y {tuple(y.shape)} does not fit [{n}, {W}]")
+        if mix is None or out is None or mix.numel() != S * S or out.numel() != S:
+            raise KernelError(f"streams_step: an output to add needs mix [{S}, {S}] and out [{S}]")
+        if rows is not None:
+            raise KernelError("streams_step: a row list goes with a read only")
+    if scale is not None and scale.numel() != W:
+        raise KernelError(f"streams_step: scale has {scale.numel()} entries, the width is {W}")
+    if read is not None and read.numel() != S:
+        raise KernelError(f"streams_step: read has {read.numel()} entries for {S} streams")
+    h = None
+    n_out = n
+    if rows is not None:
+        _i32(rows, "rows")
+        n_out = rows.numel()
+    if h_dtype is not None:
+        if norm_weight is not None and norm_weight.numel() != W:
+            raise KernelError(f"streams_step: the norm weight has {norm_weight.numel()} entries, the width is {W}")
+        h = torch.empty((n_out, W), dtype=h_dtype, device=streams.device)
+    _check(library().ia_streams_step(
+        _p(streams), _p(y), _p(y_weights), K, _p(scale), _p(mix), _p(out), _p(read), _p(norm_weight),
+        ctypes.c_float(eps), _p(h), _p(rows), n_out, S, W, _dt(y) if y is not None else 0,
+        _DT[h_dtype] if h_dtype is not None else 0, _stream()))
+    return h
+
+
+def softcap(logits: torch.Tensor, cap: float) -> torch.Tensor:
+    """cap * tanh(logits / cap), in place (32-bit)."""
+    _dev(logits); _f32(logits, "logits")
+    _check(library().ia_softcap(_p(logits), logits.numel(), ctypes.c_float(cap), _stream()))
+    return logits
+
+
+# ---- latent attention -------------------------------------------------------------------------
+
+def latent_prep(proj: torch.Tensor, *, heads: int, dim: int, rot_dim: int, rank: int, rotated: int, q_off: int,
+                down_off: int, norm_weight: torch.Tensor, eps: float, cos: Optional[torch.Tensor],
+                sin: Optional[torch.Tensor], magnitude: float, k_cache: Optional[torch.Tensor],
+                v_cache: Optional[torch.Tensor], slots: Optional[torch.Tensor], page_size: int) -> torch.Tensor:
+    """From the projections' rows to the attention's operands: the latent row is normed (32-bit) and written, with
+    the rotated shared key part behind it, to the key cache as a row and to the value cache as a column; returns
+    q [n, heads, rank + rot_dim] with the rotated parts in place at [rank:], the first `rank` features left for
+    `head_product` to fill."""
+    _dev(proj, norm_weight, cos, sin, k_cache, v_cache, slots)
+    _f32(norm_weight, "norm weight"); _f32(cos, "cos"); _f32(sin, "sin")
+    n, ld = proj.shape
+    D = rank + rot_dim
+    if norm_weight.numel() != rank:
+        raise KernelError(f"latent_prep: the norm weight has {norm_weight.numel()} entries, the rank is {rank}")
+    if rotated:
+        if cos is None or sin is None or tuple(cos.shape) != (n, rotated // 2) or cos.shape != sin.shape:
+            raise KernelError(f"latent_prep: rotary tables must be [{n}, {rotated // 2}]")
+    if slots is not None:
+        _i32(slots, "slots")
+        if k_cache is None or v_cache is None or slots.numel() != n:
+            raise KernelError("latent_prep: slots need a cache and one entry a token")
+        if (tuple(k_cache.shape[1:]) != (1, page_size, D) or tuple(v_cache.shape[1:]) != (1, D, page_size)
+                or k_cache.dtype != proj.dtype or v_cache.dtype != proj.dtype):
+            raise KernelError(f"latent_prep: cache shapes {tuple(k_cache.shape)} / {tuple(v_cache.shape)} do not fit "
+                              f"[pages, 1, {page_size}, {D}] / [pages, 1, {D}, {page_size}] {proj.dtype}")
+    q = torch.empty((n, heads, D), dtype=proj.dtype, device=proj.device)
+    _check(library().ia_latent_prep(
+        _p(q), _p(k_cache if slots is not None else None), _p(v_cache if slots is not None else None), _p(proj),
+        _p(norm_weight), _p(cos), _p(sin), _p(slots), n, heads, dim, rot_dim, rank, rotated, q_off, down_off, ld,
+        page_size, ctypes.c_float(eps), ctypes.c_float(magnitude), _dt(proj), _stream()))
+    return q
+
+
+def head_product(x: torch.Tensor, w: torch.Tensor, *, x_off: int = 0, x_head: Optional[int] = None,
+                 out: Optional[torch.Tensor] = None, o_off: int = 0, o_head: Optional[int] = None,
+                 out_dtype: Optional[torch.dtype] = None, gate: Optional[torch.Tensor] = None,
+                 g_off: int = 0) -> torch.Tensor:
+    """A product with a matrix of its own for every head: w [H, n_out, k_in]; x is 2-D, head h of row t starts at
+    x[t, x_off + h * x_head] (x_head default k_in); the result goes to out[t, o_off + h * o_head ...] (a new
+    [n, H * n_out] tensor by default).  `gate` (2-D, head h at g_off + h * n_out): times its sigmoid."""
+    _dev(x, w, out, gate)
+    H, n_out, k_in = w.shape
+    n, x_ld = x.shape
+    x_head = k_in if x_head is None else x_head
+    o_head = n_out if o_head is None else o_head
+    if out is None:
+        out = torch.empty((n, H * n_out), dtype=out_dtype or x.dtype, device=x.device)
+    if out.dim() != 2 or out.shape[0] != n:
+        raise KernelError(f"head_product: out {tuple(out.shape)} does not fit {n} rows")
+    if gate is not None and (gate.dim() != 2 or gate.shape[0] != n or gate.dtype != x.dtype):
+        raise KernelError("head_product: the gate must be 2-D rows of x's precision")
+    _check(library().ia_head_product(
+        _p(out), _p(x), _p(w), _p(gate), n, H, n_out, k_in, x_ld, x_off, x_head, out.shape[1], o_off, o_head,
+        gate.shape[1] if gate is not None else 0, g_off, _dt(x), _dt(w), _dt(out), _stream()))
+    return out
+
+
+# ---- gated linear recurrence ------------------------------------------------------------------
+
+def conv_step(x: torch.Tensor, x_off: int, width: int, taps: torch.Tensor, bias: Optional[torch.Tensor],
+              state: torch.Tensor, token_seq: torch.Tensor, cu_tokens: torch.Tensor,
+              state_slots: torch.Tensor) -> torch.Tensor:
+    """The causal convolution a channel over the step's tokens: x[:, x_off : x_off + width] -> 32-bit u
+    [n, width]; inputs before a request's portion come from rows 1.. of its state row ([slots, k, width])."""
+    _dev(x, taps, bias, state, token_seq, cu_tokens, state_slots); _f32(state, "state")
+    _i32(token_seq, "token_seq"); _i32(cu_tokens, "cu_tokens"); _i32(state_slots, "state_slots")
+    n, k = x.shape[0], taps.shape[1]
+    if (tuple(taps.shape) != (width, k) or taps.dtype != x.dtype or state.dim() != 3
+            or tuple(state.shape[1:]) != (k, width) or (bias is not None and (bias.numel() != width or bias.dtype != x.dtype))):
+        raise KernelError(f"conv_step: taps {tuple(taps.shape)} / state {tuple(state.shape)} do not fit width {width}")
+    u = torch.empty((n, width), dtype=torch.float32, device=x.device)
+    _check(library().ia_conv_step(_p(u), _p(x), _p(taps), _p(bias), _p(state), _p(token_seq), _p(cu_tokens),
+                                  _p(state_slots), n, width, k, x.shape[1], x_off, _dt(x), _stream()))
+    return u
+
+
+def rglru_scan(u: torch.Tensor, z: torch.Tensor, proj: torch.Tensor, *, branch_off: int, x_off: int,
+               bias_r: torch.Tensor, bias_i: torch.Tensor, lam: torch.Tensor, state: torch.Tensor,
+               cu_tokens: torch.Tensor, state_slots: torch.Tensor, block_width: int, decay: float) -> torch.Tensor:
+    """The recurrence over each request's tokens, from and into its state row; returns S_t * gelu_tanh(branch_t)
+    in the precision of `proj` ([n, ...]: the gelu branch at `branch_off`, the convolution's input at `x_off`).
+    z [n, 2 * width]: the gates' products before bias and sigmoid, block by block [recurrence gate | input gate]."""
+    _dev(u, z, proj, bias_r, bias_i, lam, state, cu_tokens, state_slots)
+    _f32(u, "u"); _f32(z, "z"); _f32(state, "state"); _i32(cu_tokens, "cu_tokens"); _i32(state_slots, "state_slots")
+    n, width = u.shape
+    k = state.shape[1]
+    if tuple(z.shape) != (n, 2 * width) or proj.shape[0] != n or tuple(state.shape[1:]) != (k, width):
+        raise KernelError("rglru_scan: u, z, the projections and the state do not fit each other")
+    for t in (bias_r, bias_i, lam):
+        if t.numel() != width or t.dtype != proj.dtype:
+            raise KernelError("rglru_scan: biases and decay parameters are one entry a channel in the projections' precision")
+    n_seqs = state_slots.numel()
+    out = torch.empty((n, width), dtype=proj.dtype, device=proj.device)
+    _check(library().ia_rglru_scan(
+        _p(out), _p(state), _p(u), _p(z), _p(bias_r), _p(bias_i), _p(lam), _p(proj), _p(proj), _p(cu_tokens),
+        _p(state_slots), n_seqs, width, block_width, k, ctypes.c_float(decay), proj.shape[1], branch_off,
+        proj.shape[1], x_off, _dt(proj), _stream()))
+    return out
+
+
+# ---- routed experts -----------------------------------------------------------------------------
+
+def route(h: torch.Tensor, router: torch.Tensor, top: int, scale: float, score: str = "sigmoid",
+          renormalize: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
+    """Router logits in 32-bit (router [E, width] float32), the `top` experts by score for every row:
+    (experts int32 [n, top] best first, weights float32 [n, top] = score * scale)."""
+    _dev(h, router); _f32(router, "router")
+    n, W = h.shape
+    E = router.shape[0]
+    if router.shape[1] != W or not (1 <= top <= min(E, MAX_TOP)) or E > MAX_EXPERTS or score not in SCORE_FUNCTIONS:
+        raise KernelError(f"route: router {tuple(router.shape)}, top {top}, score {score!r} (up to {MAX_EXPERTS} experts, "
+                          f"top up to {MAX_TOP}, scores {sorted(SCORE_FUNCTIONS)})")
+    sel = torch.empty((n, top), dtype=torch.int32, device=h.device)
+    weight = torch.empty((n, top), dtype=torch.float32, device=h.device)
+    _check(library().ia_route(_p(sel), _p(weight), _p(h), _p(router), n, W, E, top, ctypes.c_float(scale),
+                              SCORE_FUNCTIONS[score], int(renormalize), _dt(h), _stream()))
+    return sel, weight
+
+
+def experts_forward(h: torch.Tensor, sel: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor,
+                    limit: float, alpha: float) -> torch.Tensor:
+    """The chosen experts of every row: w_gate_up [E, 2 ff, width] (gate rows, then up rows), w_down [E, width, ff];
+    act = g' * sigmoid(alpha g') * (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit).  Returns one
+    32-bit output row a (row, k) pair, [n, top, width]; nothing is added up here."""
+    _dev(h, sel, w_gate_up, w_down); _i32(sel, "sel")
+    n, W = h.shape
+    top = sel.shape[1]
+    E, ff2, W2 = w_gate_up.shape
+    ff = ff2 // 2
+    if (W2 != W or ff2 != 2 * ff or tuple(w_down.shape) != (E, W, ff) or w_gate_up.dtype != h.dtype
+            or w_down.dtype != h.dtype or sel.shape[0] != n or E > MAX_EXPERTS):
+        raise KernelError(f"experts: weights {tuple(w_gate_up.shape)} / {tuple(w_down.shape)} do not fit rows {tuple(h.shape)}")
+    pairs = n * top
+    tiles = -(-pairs // ROW_TILE) + min(E, pairs)
+    lib = library()
+    plan = torch.empty((pairs + 3 * tiles + 1,), dtype=torch.int32, device=h.device)
+    order, t_exp, t_first, t_rows, meta = (plan[:pairs], plan[pairs:pairs + tiles], plan[pairs + tiles:pairs + 2 * tiles],
+                                           plan[pairs + 2 * tiles:pairs + 3 * tiles], plan[pairs + 3 * tiles:])
+    _check(lib.ia_route_plan(_p(order), _p(t_exp), _p(t_first), _p(t_rows), _p(meta), _p(sel), pairs, E, _stream()))
+    act = torch.empty((pairs, ff), dtype=h.dtype, device=h.device)
+    _check(lib.ia_experts_gate_up(_p(act), _p(h), _p(w_gate_up), _p(order), _p(t_exp), _p(t_first), _p(t_rows), _p(meta),
+                                  pairs, E, top, W, ff, ctypes.c_float(limit), ctypes.c_float(alpha), _dt(h), _stream()))
+    y = torch.empty((n, top, W), dtype=torch.float32, device=h.device)
+    _check(lib.ia_experts_down(_p(y), _p(act), _p(w_down), _p(order), _p(t_exp), _p(t_first), _p(t_rows), _p(meta), pairs,
+                               E, W, ff, _dt(h), _stream()))
+    return y

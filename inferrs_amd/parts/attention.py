@@ -76,6 +76,8 @@ class Attention(Mixer):
             self.q_norm_w = self.k_norm_w = None
             self.norm_eps, self.norm_add_one = 0.0, False
         self.position = part_class("position", spec.position)(spec.position, {}, dtype, device)
+        if getattr(self.position, "magnitude", 1.0) != 1.0:
+            raise SpecError("attention: a rotation law that scales cos and sin is not taken by this mixer's kernels")
 
     def load_notes(self, page_size: int):
         """What the log should say once when a model with this part is set up: a decode step that cannot take the

@@ -65,3 +65,14 @@ class LinearHead(Head):
 
     def forward(self, rows: torch.Tensor) -> torch.Tensor:
         return ops.linear(rows, self.weight, torch.float32)
+
+
+@register_head("capped_lm_head")
+class CappedHead(LinearHead):
+    """A product with the head's matrix, then cap * tanh(logits / cap) (`spec.cap` None: no cap)."""
+
+    def forward(self, rows: torch.Tensor) -> torch.Tensor:
+        logits = super().forward(rows)
+        if self.spec.cap is not None:
+            ops.softcap(logits, float(self.spec.cap))
+        return logits

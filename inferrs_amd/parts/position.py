@@ -2,6 +2,7 @@
 (`inferrs-models/src/models/attention_utils.rs:186-216`); "none": nothing."""
 from __future__ import annotations
 
+import math
 from typing import Optional, Tuple
 
 import numpy as np
@@ -30,8 +31,34 @@ def linear_scaling(inv_freq: np.ndarray, factor: float) -> np.ndarray:
     return (inv_freq / np.float32(factor)).astype(np.float32)
 
 
-# name of a scaling law -> (inverse frequencies, factor) -> inverse frequencies; another law is another entry
-SCALING_LAWS = {"linear": linear_scaling}
+def yarn_scaling(inv_freq: np.ndarray, factor: float, original: float, fast: float, slow: float, *, theta: float,
+                 rot_dim: int):
+    """Pairs that turn fast keep their frequency, slow ones are divided by `factor`, a linear ramp between the pair
+    that makes `fast` turns over `original` positions and the one that makes `slow`: with
+    pair(t) = rot_dim ln(original / (2 pi t)) / (2 ln theta), lo = max(floor(pair(fast)), 0),
+    hi = min(ceil(pair(slow)), rot_dim - 1), ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1),
+    f_i <- f_i / factor * ramp_i + f_i (1 - ramp_i).  cos and sin are multiplied by 0.1 ln(factor) + 1.
+    Returns (frequencies, that factor).  (Peng et al., "YaRN: Efficient Context Window Extension of Large
+    Language Models".)"""
+    if not (factor > 0.0 and original > 0.0 and fast > 0.0 and slow > 0.0 and theta > 1.0):
+        raise SpecError(f"rotary scaling 'yarn' needs positive numbers, got factor={factor} original={original} "
+                        f"fast={fast} slow={slow} base={theta}")
+
+    def pair(turns: float) -> float:
+        return rot_dim * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(theta))
+
+    lo = max(math.floor(pair(fast)), 0)
+    hi = min(math.ceil(pair(slow)), rot_dim - 1)
+    i = np.arange(inv_freq.shape[0], dtype=np.float64)
+    ramp = np.clip((i - lo) / max(hi - lo, 0.001), 0.0, 1.0)
+    f = inv_freq.astype(np.float64)
+    return (f / factor * ramp + f * (1.0 - ramp)).astype(np.float32), 0.1 * math.log(factor) + 1.0
+
+
+# name of a scaling law -> (inverse frequencies, the law's numbers) -> inverse frequencies, or (inverse frequencies,
+# factor on cos and sin); a law that needs the base and the rotated size says so in SCALING_NEEDS_GEOMETRY
+SCALING_LAWS = {"linear": linear_scaling, "yarn": yarn_scaling}
+SCALING_NEEDS_GEOMETRY = {"yarn"}
 
 
 @register_position("rope")
@@ -47,11 +74,17 @@ class Rotary(Position):
         self.rot_dim = spec.rot_dim
         self.interleaved = spec.pairing == "interleaved"
         inv_freq = inverse_frequencies(spec.theta, spec.rot_dim)
+        self.magnitude = 1.0             # cos and sin are multiplied by this (the kernels that rotate take it)
         if spec.scaling is not None:
-            law, factor = spec.scaling
+            law, numbers = spec.scaling[0], [float(v) for v in spec.scaling[1:]]
             if law not in SCALING_LAWS:
                 raise SpecError(f"rotary scaling {law!r} has no entry (known: {sorted(SCALING_LAWS)})")
-            inv_freq = SCALING_LAWS[law](inv_freq, float(factor))
+            extra = dict(theta=float(spec.theta), rot_dim=spec.rot_dim) if law in SCALING_NEEDS_GEOMETRY else {}
+            scaled = SCALING_LAWS[law](inv_freq, *numbers, **extra)
+            if isinstance(scaled, tuple):
+                inv_freq, self.magnitude = scaled[0], float(scaled[1])
+            else:
+                inv_freq = scaled
         self.inv_freq = torch.from_numpy(inv_freq).to(device)
 
     def table(self, positions: torch.Tensor) -> Optional[Tuple[torch.Tensor, torch.Tensor]]:
@@ -64,6 +97,7 @@ class NoPosition(Position):
 
     rot_dim = 0
     interleaved = False
+    magnitude = 1.0
 
     def __init__(self, spec, tensors, dtype, device):
         self.spec = spec

@@ -5,8 +5,9 @@ The reference has no random-weight mode for this model (candle's
 tensor has a seed of its own from (seed, tensor name) and each element is a
 function of (that seed, its index) alone, so values do not depend on which other
 tensors exist, on the order of filling or on where they are filled (host or
-GPU): matrices N(0, 0.02), norm weights 1 + N(0, 0.1), rounded to 32-bit and
-then to the storage precision.
+GPU): matrices N(0, 0.02), norm weights 1 + N(0, 0.1), small square matrices that
+mix residual streams identity + N(0, 0.1), rounded to 32-bit and then to the storage
+precision.
 """
 from __future__ import annotations
 
@@ -90,12 +91,14 @@ def random_tensors(expected: Mapping[str, TensorSpec], seed: int,
             out[name] = torch.from_numpy(table_values(n_elements(spec.shape), _tensor_seed(seed, name), spec.high)
                                          ).reshape(spec.shape).to(device)
             continue
-        mean, std = (1.0, NORM_STD) if spec.init == "norm" else (0.0, MATRIX_STD)
+        mean, std = (1.0, NORM_STD) if spec.init == "norm" else (0.0, NORM_STD) if spec.init == "eye" else (0.0, MATRIX_STD)
         tseed = _tensor_seed(seed, name)
         if on_gpu:
             out[name] = ops.fill_normal(spec.shape, tseed, mean, std, dtype, device)
         else:
             out[name] = torch.from_numpy(normal_values(n_elements(spec.shape), tseed, mean, std)).reshape(spec.shape).to(dtype)
+        if spec.init == "eye":                   # a square matrix near the identity
+            out[name] = (out[name].float() + torch.eye(spec.shape[0], device=out[name].device)).to(out[name].dtype)
     return out
 
 
