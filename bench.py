@@ -345,6 +345,79 @@ def workload_main(args, raw, engine_factory) -> int:
     return 0
 
 
+# ---- the Buketar design beside the dense decoder at equal size (`--design buketar`) ---------------------------
+# Layer sizes in the range of real models of its kind: latent attention with a cached row of 256 (latent 192 + 64
+# rotated), recurrent blocks as wide as the model, 32 small experts of which a token runs 4.  The dense twin has the
+# same width and number of layers, as many attention heads of size 128 as fill the width, and a feed-forward as large
+# as the experts that a token runs (top x ff), so that a token costs about the same products in both.
+def buketar_shape(width: int, layers: int, heads: int, experts: int, top: int, ff: int, vocab: int = 32768):
+    att = {"type": "latent_attention",
+           "mixer": {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 192, "scale": 192 ** -0.5,
+                     "rot": {"base": 10000.0, "dims": 64, "scaling": {"factor": 8.0, "original": 4096, "fast": 32.0, "slow": 1.0}}}}
+    rec = {"type": "rglru", "mixer": {"width": width, "blocks": max(1, width // 256), "conv": 4}}
+    mlp = {"kind": "moe", "expert": {"ff": ff, "limit": 7.0}, "router": {"experts": experts, "top": top, "scale": 1.0}}
+    pattern = [rec, rec, att]
+    return {"architecture": "Buketar", "vocab": vocab, "width": width, "norm": {"eps": 1e-6}, "streams": 2,
+            "logit_softcap": 30.0, "layers": [dict(pattern[i % 3], mlp=mlp) for i in range(layers)]}
+
+
+BUKETAR_SHAPES = {"1k": dict(width=1024, layers=12, heads=8, experts=32, top=4, ff=768),
+                  "2k": dict(width=2048, layers=12, heads=16, experts=32, top=4, ff=1536),
+                  "4k": dict(width=4096, layers=6, heads=32, experts=32, top=4, ff=3072)}
+
+
+def dense_twin(b: dict, vocab: int = 32768) -> dict:
+    return dict(QWEN3_8B, vocab_size=vocab, hidden_size=b["width"], intermediate_size=b["top"] * b["ff"],
+                num_hidden_layers=b["layers"], num_attention_heads=b["width"] // 128, num_key_value_heads=max(1, b["width"] // 512),
+                tie_word_embeddings=False)
+
+
+# what a kernel of the new design moves or multiplies at least, against the memory or the matrix roof: entry point ->
+# the like kernel of the dense decoder that it is compared with
+LIKE_KERNEL = {"streams_step": "add_rmsnorm", "latent_prep": "qk_rope_kv", "head_product": "vendor_gemm",
+               "experts_gate_up": "vendor_gemm", "experts_down": "vendor_gemm", "rglru_scan": "add_rmsnorm",
+               "conv_step": "add_rmsnorm", "route": "rmsnorm", "route_plan": "rmsnorm", "softcap": "rmsnorm"}
+
+
+def design_main(args) -> int:
+    """Prefill and decode throughput of the Buketar design at a few layer sizes beside the dense decoder at equal
+    size (random weights), and the time of every kernel of one prefill and one decode step of both."""
+    import torch
+    from inferrs_amd.config import Qwen3Config
+    from inferrs_amd.config.buketar import BuketarConfig
+    from inferrs_amd.engine import Engine
+    batch, context, prompt = args.batch, min(args.context, 2048), args.prefill_tokens
+    records = {}
+    for name in (args.design_shapes.split(",") if args.design_shapes else sorted(BUKETAR_SHAPES)):
+        b = BUKETAR_SHAPES[name]
+        raw_new, raw_old = buketar_shape(**b), dense_twin(b)
+        rec = {}
+        for label, config, vocab in (("buketar", BuketarConfig.from_dict(raw_new), raw_new["vocab"]),
+                                     ("dense", Qwen3Config.from_dict(raw_old), raw_old["vocab_size"])):
+            pages = batch * (-(-context // PAGE) + 1) + -(-prompt // PAGE) + 8
+            note(f"{name} {label}: random weights, {pages} pages")
+            engine = Engine.from_random(config, seed=0, dtype=args.dtype, page_size=PAGE, num_pages=pages, max_seqs=batch + 1)
+            fill_storage(engine)
+            times = time_prefill(engine, prompt, args.runs, vocab)
+            p_mean, p_std = mean_std(times)
+            elapsed, _ = time_decode(engine, batch, context, args.steps, args.warmup, decode_run=args.decode_run)
+            one, _ = time_decode(engine, 1, context, args.steps, args.warmup, decode_run=args.decode_run)
+            rec[label] = {"weights_gb": round(engine.model.weight_bytes() / 1e9, 3),
+                          "prefill_tok_s": round(prompt / p_mean, 1), "prefill_ms": round(p_mean * 1e3, 3),
+                          f"decode_b{batch}_tok_s": round(batch * args.steps / elapsed, 1),
+                          f"decode_b{batch}_ms_per_step": round(elapsed / args.steps * 1e3, 3),
+                          "decode_b1_tok_s": round(args.steps / one, 1),
+                          "kernels": kernel_breakdown(engine, batch, context, prompt, vocab)}
+            del engine
+            torch.cuda.empty_cache()
+        records[name] = rec
+    print(json.dumps({"metric": "design_throughput", "design": "Buketar", "beside": "Qwen3 dense at equal width, layers and "
+                      "feed-forward products a token", "dtype": args.dtype, "data": "synthetic", "batch": batch, "context": context,
+                      "prefill_tokens": prompt, "steps": args.steps, "warmup": args.warmup, "like_kernel": LIKE_KERNEL,
+                      "shapes": records}))
+    return 0
+
+
 def note(msg: str) -> None:
     """Progress goes to stderr; the one JSON line is all that stdout carries."""
     print(f"[bench] {msg}", file=sys.stderr, flush=True)
@@ -377,10 +450,17 @@ def main() -> int:
                     help="workloads: cut prompt portions so that a step's tokens are a multiple of this (0: off)")
     ap.add_argument("--decode-run", type=int, default=8,
                     help="decode steps that the serving loop queues on the GPU at once (1: one at a time)")
+    ap.add_argument("--design", default=None, choices=["buketar"],
+                    help="instead of the headline: prefill and decode throughput of this design at a few layer sizes "
+                         "beside the dense decoder at equal size, with every kernel's time")
+    ap.add_argument("--design-shapes", default=None, help="with --design: the sizes to run, with commas (default: all)")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+
+    if args.design:
+        return design_main(args)
 
     import torch
     from inferrs_amd.config import Qwen3Config

@@ -154,7 +154,8 @@ int ia_head_product(void* out, const void* x, const void* w, const void* gate, i
                     long long g_ld, int g_off, int x_dtype, int w_dtype, int out_dtype, hipStream_t stream);
 
 // ---- gated linear recurrence behind a short convolution (recurrence.hip) ----------------------------------------
-int ia_conv_step(float* u, const void* x, const void* taps, const void* bias, const float* state,
+// u_lo: null, or a bfloat16 copy of u (for products that take it in that precision)
+int ia_conv_step(float* u, void* u_lo, const void* x, const void* taps, const void* bias, const float* state,
                  const int* token_seq, const int* cu_tokens, const int* state_slots, int n, int width, int k,
                  long long x_ld, int x_off, int dtype, hipStream_t stream);
 int ia_rglru_scan(void* out, float* state, const float* u, const float* z, const void* bias_r,
@@ -162,11 +163,19 @@ int ia_rglru_scan(void* out, float* state, const float* u, const float* z, const
                   const int* cu_tokens, const int* state_slots, int n_seqs, int width, int bw, int k,
                   float decay, long long b_ld, int b_off, long long x_ld, int x_off, int dtype,
                   hipStream_t stream);
+// the same for long portions: chunks of 64 tokens side by side (rounding apart, the same result); `work` holds
+// ia_rglru_chunked_workspace(...) 32-bit words
+long long ia_rglru_chunked_workspace(int n, int n_seqs, int width);
+int ia_rglru_scan_chunked(void* out, float* state, float* work, const float* u, const float* z,
+                          const void* bias_r, const void* bias_i, const void* lam, const void* branch,
+                          const void* x, const int* cu_tokens, const int* state_slots, int n, int n_seqs,
+                          int width, int bw, int k, float decay, long long b_ld, int b_off, long long x_ld,
+                          int x_off, int dtype, hipStream_t stream);
 
 // ---- routed experts (experts.hip) --------------------------------------------------------------------------------
 // score_fn: 0 sigmoid, 1 softmax over all experts
-int ia_route(int* sel, float* weight, const void* h, const float* router, int n, int W, int E, int top,
-             float scale, int score_fn, int renorm, int dtype, hipStream_t stream);
+int ia_route(int* sel, float* weight, const float* logits, int n, int E, int top, float scale, int score_fn,
+             int renorm, hipStream_t stream);
 int ia_route_tiles(int pairs, int E);
 int ia_route_plan(int* order, int* tile_expert, int* tile_first, int* tile_rows, int* meta, const int* sel,
                   int pairs, int E, hipStream_t stream);

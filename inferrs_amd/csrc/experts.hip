@@ -1,8 +1,9 @@
 // Routed experts: a router scores every expert for a token, the `top` best are run and their outputs added up
 // with the scores as weights.
 //
-//   route      a wave a token: router logits in 32-bit, scores = sigmoid (or softmax), the top experts by score
-//              (ties: the lower index), weights = score * scale (optionally renormalised over the chosen).
+//   route      a wave a token, from the router's 32-bit logits (a product of the 32-bit path): scores = sigmoid (or
+//              softmax), the top experts by score (ties: the lower index), weights = score * scale (optionally
+//              renormalised over the chosen).
 //   plan       one block: the (token, k) pairs ordered by expert, and a table of row tiles (expert, first pair, rows),
 //              all on the device: the host never learns how many tokens an expert got.
 //   gate_up    tile by tile: rows gathered by pair, act(gate, up) in the epilogue.
@@ -11,29 +12,22 @@
 #include "api.h"
 #include "common.h"
 #include "tile_fma.h"
+#include "tile_mfma.h"
 
 #define IA_MAX_EXPERTS 256
 #define IA_MAX_TOP 16
 
 enum { IA_SCORE_SIGMOID = 0, IA_SCORE_SOFTMAX = 1 };
 
-template <typename T>
 __global__ __launch_bounds__(64) void route_kernel(int* __restrict__ sel, float* __restrict__ weight,
-                                                   const T* __restrict__ h, const float* __restrict__ wr, int n, int W,
-                                                   int E, int top, float scale, int score_fn, int renorm) {
+                                                   const float* __restrict__ logits, int n, int E, int top, float scale,
+                                                   int score_fn, int renorm) {
     const int t = blockIdx.x, lane = threadIdx.x;
-    const T* row = h + (long long)t * W;
     float z[IA_MAX_EXPERTS / IA_WAVE];             // expert e lives in lane e % 64, register e / 64
 #pragma unroll
-    for (int q = 0; q < IA_MAX_EXPERTS / IA_WAVE; ++q) z[q] = -INFINITY;
-    for (int e = 0; e < E; ++e) {
-        const float* w = wr + (long long)e * W;
-        float acc = 0.f;
-        for (int c = lane; c < W; c += IA_WAVE) acc = fmaf(ld(row + c), w[c], acc);
-        acc = wave_sum(acc);
-#pragma unroll
-        for (int q = 0; q < IA_MAX_EXPERTS / IA_WAVE; ++q)
-            if (e == q * IA_WAVE + lane) z[q] = acc;
+    for (int q = 0; q < IA_MAX_EXPERTS / IA_WAVE; ++q) {
+        const int e = q * IA_WAVE + lane;
+        z[q] = e < E ? logits[(long long)t * E + e] : -INFINITY;
     }
     float zmax = -INFINITY, denom = 1.f;
     if (score_fn == IA_SCORE_SOFTMAX) {
@@ -171,16 +165,74 @@ __global__ __launch_bounds__(256) void experts_down_kernel(float* __restrict__ y
     }
 }
 
-extern "C" int ia_route(int* sel, float* weight, const void* h, const float* router, int n, int W, int E, int top,
-                        float scale, int score_fn, int renorm, int dtype, hipStream_t stream) {
-    IA_CHECK(n >= 0 && W > 0 && E >= 1 && E <= IA_MAX_EXPERTS && top >= 1 && top <= E && top <= IA_MAX_TOP,
-             "route: n=%d width=%d experts=%d (up to %d) top=%d (up to %d)", n, W, E, IA_MAX_EXPERTS, top, IA_MAX_TOP);
+// The same two products on the matrix cores (bfloat16; widths in steps of 8).
+__global__ __launch_bounds__(256) void experts_gate_up_mfma_kernel(bf16_t* __restrict__ act, const bf16_t* __restrict__ h,
+                                                                   const bf16_t* __restrict__ w_gu,
+                                                                   const int* __restrict__ order,
+                                                                   const int* __restrict__ tile_expert,
+                                                                   const int* __restrict__ tile_first,
+                                                                   const int* __restrict__ tile_rows,
+                                                                   const int* __restrict__ meta, int top, int W, int ff,
+                                                                   float limit, float alpha) {
+    __shared__ TileSharedMfma sh;
+    const int tile = blockIdx.y;
+    if (tile >= meta[0]) return;
+    const int e = tile_expert[tile], first = tile_first[tile], rows = tile_rows[tile], col0 = blockIdx.x * IA_MN;
+    tm_f32x4 g[2], u[2];
+    auto xrow = [&](int i) -> const bf16_t* { return i < rows ? h + (long long)(order[first + i] / top) * W : nullptr; };
+    const bf16_t* wg = w_gu + ((long long)e * 2 * ff + col0) * W;
+    tile_product_mfma<true>(g, u, sh, xrow, wg, wg + (long long)ff * W, ff - col0, W, W);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+        const int i = 16 * rt + (lane & 15);
+        if (i >= rows) continue;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int j = col0 + 16 * wave + 4 * (lane >> 4) + q;
+            if (j >= ff) continue;
+            const float gv = fminf(g[rt][q], limit), uv = fminf(fmaxf(u[rt][q], -limit), limit);
+            st(act + (long long)(first + i) * ff + j, gv / (1.0f + expf(-alpha * gv)) * (uv + 1.0f));
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void experts_down_mfma_kernel(float* __restrict__ y, const bf16_t* __restrict__ act,
+                                                                const bf16_t* __restrict__ w_down,
+                                                                const int* __restrict__ order,
+                                                                const int* __restrict__ tile_expert,
+                                                                const int* __restrict__ tile_first,
+                                                                const int* __restrict__ tile_rows,
+                                                                const int* __restrict__ meta, int W, int ff) {
+    __shared__ TileSharedMfma sh;
+    const int tile = blockIdx.y;
+    if (tile >= meta[0]) return;
+    const int e = tile_expert[tile], first = tile_first[tile], rows = tile_rows[tile], col0 = blockIdx.x * IA_MN;
+    tm_f32x4 acc[2], unused[2];
+    auto xrow = [&](int i) -> const bf16_t* { return i < rows ? act + (long long)(first + i) * ff : nullptr; };
+    const bf16_t* wd = w_down + ((long long)e * W + col0) * ff;
+    tile_product_mfma<false>(acc, unused, sh, xrow, wd, wd, W - col0, ff, ff);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+        const int i = 16 * rt + (lane & 15);
+        if (i >= rows) continue;
+        const long long pair = order[first + i];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int c = col0 + 16 * wave + 4 * (lane >> 4) + q;
+            if (c < W) y[pair * W + c] = acc[rt][q];
+        }
+    }
+}
+
+extern "C" int ia_route(int* sel, float* weight, const float* logits, int n, int E, int top, float scale, int score_fn,
+                        int renorm, hipStream_t stream) {
+    IA_CHECK(n >= 0 && E >= 1 && E <= IA_MAX_EXPERTS && top >= 1 && top <= E && top <= IA_MAX_TOP,
+             "route: n=%d experts=%d (up to %d) top=%d (up to %d)", n, E, IA_MAX_EXPERTS, top, IA_MAX_TOP);
     IA_CHECK(score_fn == IA_SCORE_SIGMOID || score_fn == IA_SCORE_SOFTMAX, "route: unknown score function %d", score_fn);
     if (n == 0) return 0;
-    if (dtype == IA_F32)
-        route_kernel<float><<<n, 64, 0, stream>>>(sel, weight, (const float*)h, router, n, W, E, top, scale, score_fn, renorm);
-    else
-        route_kernel<bf16_t><<<n, 64, 0, stream>>>(sel, weight, (const bf16_t*)h, router, n, W, E, top, scale, score_fn, renorm);
+    route_kernel<<<n, 64, 0, stream>>>(sel, weight, logits, n, E, top, scale, score_fn, renorm);
     IA_LAUNCH_CHECK("route");
     return 0;
 }
@@ -203,7 +255,10 @@ extern "C" int ia_experts_gate_up(void* act, const void* h, const void* w_gu, co
     if (pairs == 0) return 0;
     const dim3 grid((ff + IA_TN - 1) / IA_TN, ia_route_tiles(pairs, E));
     IA_CHECK(grid.y <= 65535, "experts_gate_up: %u row tiles are more than a grid takes", grid.y);
-    if (dtype == IA_F32)
+    if (dtype == IA_BF16 && W % 8 == 0 && tile_mfma_aligned(h) && tile_mfma_aligned(w_gu))
+        experts_gate_up_mfma_kernel<<<grid, 256, 0, stream>>>((bf16_t*)act, (const bf16_t*)h, (const bf16_t*)w_gu, order, tile_expert,
+                                                              tile_first, tile_rows, meta, top, W, ff, limit, alpha);
+    else if (dtype == IA_F32)
         experts_gate_up_kernel<float><<<grid, 256, 0, stream>>>((float*)act, (const float*)h, (const float*)w_gu, order,
                                                                 tile_expert, tile_first, tile_rows, meta, top, W, ff, limit, alpha);
     else
@@ -220,7 +275,10 @@ extern "C" int ia_experts_down(float* y, const void* act, const void* w_down, co
     if (pairs == 0) return 0;
     const dim3 grid((W + IA_TN - 1) / IA_TN, ia_route_tiles(pairs, E));
     IA_CHECK(grid.y <= 65535, "experts_down: %u row tiles are more than a grid takes", grid.y);
-    if (dtype == IA_F32)
+    if (dtype == IA_BF16 && ff % 8 == 0 && tile_mfma_aligned(act) && tile_mfma_aligned(w_down))
+        experts_down_mfma_kernel<<<grid, 256, 0, stream>>>(y, (const bf16_t*)act, (const bf16_t*)w_down, order, tile_expert, tile_first,
+                                                           tile_rows, meta, W, ff);
+    else if (dtype == IA_F32)
         experts_down_kernel<float><<<grid, 256, 0, stream>>>(y, (const float*)act, (const float*)w_down, order, tile_expert,
                                                              tile_first, tile_rows, meta, W, ff);
     else

@@ -11,6 +11,7 @@
 #include "api.h"
 #include "common.h"
 #include "tile_fma.h"
+#include "tile_mfma.h"
 
 // proj[t] = [.. q (H x (d + r)) at q_off .. | down (rank + r) at down_off ..]; q_out [n, H, rank + r] gets the
 // rotated parts at [rank, rank + r).  Of a rotated part the first `rd` features turn (i paired with i + rd / 2), the
@@ -135,8 +136,41 @@ __global__ __launch_bounds__(256) void head_product_kernel(
     }
 }
 
-// dtypes: 0 float32, 1 bfloat16 (x and gate share one).  Combinations built: x and w and out alike; x float32 with w
-// bfloat16 and out float32 (32-bit rows against stored bfloat16 matrices).
+// The same on the matrix cores: bfloat16 rows and matrices, k_in and every offset a multiple of 8.
+template <typename TO>
+__global__ __launch_bounds__(256) void head_product_mfma_kernel(
+    TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const bf16_t* __restrict__ gate, int n,
+    int n_out, int k_in, long long x_ld, int x_off, int x_head, long long o_ld, int o_off, int o_head, long long g_ld,
+    int g_off) {
+    __shared__ TileSharedMfma sh;
+    const int h = blockIdx.z, row0 = blockIdx.y * IA_MM, col0 = blockIdx.x * IA_MN;
+    tm_f32x4 acc[2], unused[2];
+    const bf16_t* xb = x + x_off + (long long)h * x_head;
+    auto xrow = [&](int i) -> const bf16_t* { return row0 + i < n ? xb + (long long)(row0 + i) * x_ld : nullptr; };
+    const bf16_t* wt = w + ((long long)h * n_out + col0) * k_in;
+    tile_product_mfma<false>(acc, unused, sh, xrow, wt, wt, n_out - col0, k_in, k_in);
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+#pragma unroll
+    for (int rt = 0; rt < 2; ++rt) {
+        const int t = row0 + 16 * rt + (lane & 15);
+        if (t >= n) continue;
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int j = col0 + 16 * wave + 4 * (lane >> 4) + q;
+            if (j >= n_out) continue;
+            float v = acc[rt][q];
+            if (gate != nullptr) {
+                const float g = ld(gate + (long long)t * g_ld + g_off + (long long)h * n_out + j);
+                v = v / (1.0f + expf(-g));
+            }
+            st(out + (long long)t * o_ld + o_off + (long long)h * o_head + j, v);
+        }
+    }
+}
+
+// dtypes: 0 float32, 1 bfloat16 (x and gate share one).  Combinations built: x and w and out alike; 32-bit results of
+// bfloat16 matrices with rows in either precision.  bfloat16 rows and matrices whose sizes and offsets are multiples of
+// 8 run on the matrix cores, the rest on the vector units.
 extern "C" int ia_head_product(void* out, const void* x, const void* w, const void* gate, int n, int H, int n_out,
                                int k_in, long long x_ld, int x_off, int x_head, long long o_ld, int o_off, int o_head,
                                long long g_ld, int g_off, int x_dtype, int w_dtype, int out_dtype, hipStream_t stream) {
@@ -153,9 +187,20 @@ extern "C" int ia_head_product(void* out, const void* x, const void* w, const vo
     head_product_kernel<TX, TW, TO><<<grid, 256, 0, stream>>>((TO*)out, (const TX*)x, (const TW*)w, (const TX*)gate, n, \
                                                               n_out, k_in, x_ld, x_off, x_head, o_ld, o_off, o_head,  \
                                                               g_ld, g_off)
-    if (x_dtype == IA_F32 && w_dtype == IA_F32 && out_dtype == IA_F32) IA_LAUNCH(float, float, float);
+    const bool cores = x_dtype == IA_BF16 && w_dtype == IA_BF16 && k_in % 8 == 0 && x_ld % 8 == 0 && x_off % 8 == 0 &&
+                       x_head % 8 == 0 && tile_mfma_aligned(x) && tile_mfma_aligned(w);
+    if (cores && out_dtype == IA_BF16)
+        head_product_mfma_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, (const bf16_t*)w,
+                                                                   (const bf16_t*)gate, n, n_out, k_in, x_ld, x_off, x_head,
+                                                                   o_ld, o_off, o_head, g_ld, g_off);
+    else if (cores && out_dtype == IA_F32)
+        head_product_mfma_kernel<float><<<grid, 256, 0, stream>>>((float*)out, (const bf16_t*)x, (const bf16_t*)w,
+                                                                  (const bf16_t*)gate, n, n_out, k_in, x_ld, x_off, x_head,
+                                                                  o_ld, o_off, o_head, g_ld, g_off);
+    else if (x_dtype == IA_F32 && w_dtype == IA_F32 && out_dtype == IA_F32) IA_LAUNCH(float, float, float);
     else if (x_dtype == IA_BF16 && w_dtype == IA_BF16 && out_dtype == IA_BF16) IA_LAUNCH(bf16_t, bf16_t, bf16_t);
     else if (x_dtype == IA_F32 && w_dtype == IA_BF16 && out_dtype == IA_F32) IA_LAUNCH(float, bf16_t, float);
+    else if (x_dtype == IA_BF16 && w_dtype == IA_BF16 && out_dtype == IA_F32) IA_LAUNCH(bf16_t, bf16_t, float);
     else {
         ia_set_error("head_product: no kernel for the dtypes x=%d w=%d out=%d", x_dtype, w_dtype, out_dtype);
         return 1;

@@ -11,7 +11,7 @@
 
 // u [n, width] (32-bit) of the step's tokens; reads the inputs that precede a request's portion from its state row.
 template <typename T>
-__global__ void conv_step_kernel(float* __restrict__ u, const T* __restrict__ x, const T* __restrict__ taps,
+__global__ void conv_step_kernel(float* __restrict__ u, bf16_t* __restrict__ u_lo, const T* __restrict__ x, const T* __restrict__ taps,
                                  const T* __restrict__ bias, const float* __restrict__ state,
                                  const int* __restrict__ token_seq, const int* __restrict__ cu_tokens,
                                  const int* __restrict__ state_slots, int width, int k, long long x_ld, int x_off,
@@ -31,6 +31,7 @@ __global__ void conv_step_kernel(float* __restrict__ u, const T* __restrict__ x,
         acc = fmaf(ld(taps + (long long)c * k + j), v, acc);
     }
     u[i] = acc;
+    if (u_lo != nullptr) st(u_lo + i, acc);
 }
 
 // One thread a (request, channel) walks the request's tokens in order.  z [n, 2 * width] holds, block by block,
@@ -76,7 +77,7 @@ __global__ void rglru_scan_kernel(T* __restrict__ out, float* __restrict__ state
     }
 }
 
-extern "C" int ia_conv_step(float* u, const void* x, const void* taps, const void* bias, const float* state,
+extern "C" int ia_conv_step(float* u, void* u_lo, const void* x, const void* taps, const void* bias, const float* state,
                             const int* token_seq, const int* cu_tokens, const int* state_slots, int n, int width, int k,
                             long long x_ld, int x_off, int dtype, hipStream_t stream) {
     IA_CHECK(n >= 0 && width > 0 && k >= 1 && x_off >= 0 && x_off + width <= x_ld, "conv_step: bad sizes n=%d width=%d taps=%d",
@@ -85,10 +86,10 @@ extern "C" int ia_conv_step(float* u, const void* x, const void* taps, const voi
     if (total == 0) return 0;
     const int blocks = (int)((total + 255) / 256);
     if (dtype == IA_F32)
-        conv_step_kernel<float><<<blocks, 256, 0, stream>>>(u, (const float*)x, (const float*)taps, (const float*)bias, state,
+        conv_step_kernel<float><<<blocks, 256, 0, stream>>>(u, (bf16_t*)u_lo, (const float*)x, (const float*)taps, (const float*)bias, state,
                                                             token_seq, cu_tokens, state_slots, width, k, x_ld, x_off, total);
     else
-        conv_step_kernel<bf16_t><<<blocks, 256, 0, stream>>>(u, (const bf16_t*)x, (const bf16_t*)taps, (const bf16_t*)bias,
+        conv_step_kernel<bf16_t><<<blocks, 256, 0, stream>>>(u, (bf16_t*)u_lo, (const bf16_t*)x, (const bf16_t*)taps, (const bf16_t*)bias,
                                                              state, token_seq, cu_tokens, state_slots, width, k, x_ld, x_off,
                                                              total);
     IA_LAUNCH_CHECK("conv_step");
@@ -116,5 +117,145 @@ extern "C" int ia_rglru_scan(void* out, float* state, const float* u, const floa
                                                            (const bf16_t*)x, cu_tokens, state_slots, width, bw, k, decay, b_ld,
                                                            b_off, x_ld, x_off);
     IA_LAUNCH_CHECK("rglru_scan");
+    return 0;
+}
+
+// ---- the same recurrence for long portions: in chunks of 64 tokens side by side -----------------------------------
+// S_t = a_t S_(t-1) + b_t is linear in the state a chunk starts from: with L_t the state reached from zero at the
+// chunk's start and A_t the product of the chunk's decays up to t, S_t = L_t + A_t * S_in(chunk).  Three kernels:
+// every chunk from zero (a thread a chunk and channel); a request's chunks in order (a thread a request and channel:
+// S_in of the next chunk = L_end + A_end * S_in, then the state row and the convolution's last inputs); every token
+// from its chunk's S_in.  The result differs from the token-by-token walk by rounding only.
+#define IA_SCAN_CHUNK 64
+
+// chunk g of the step -> its request and token range; requests own ceil(tokens / 64) chunks each, in order
+__device__ __forceinline__ bool scan_chunk(const int* __restrict__ cu, int n_seqs, int g, int& seq, int& begin, int& end) {
+    int at = 0;
+    for (int s = 0; s < n_seqs; ++s) {
+        const int first = cu[s], last = cu[s + 1];
+        const int nc = (last - first + IA_SCAN_CHUNK - 1) / IA_SCAN_CHUNK;
+        if (g < at + nc) {
+            seq = s;
+            begin = first + (g - at) * IA_SCAN_CHUNK;
+            end = begin + IA_SCAN_CHUNK < last ? begin + IA_SCAN_CHUNK : last;
+            return true;
+        }
+        at += nc;
+    }
+    return false;
+}
+
+template <typename T>
+__global__ void rglru_chunks_kernel(float* __restrict__ loc, float* __restrict__ cum, float* __restrict__ chunk_a,
+                                    float* __restrict__ chunk_l, int* __restrict__ token_chunk, const float* __restrict__ u,
+                                    const float* __restrict__ z, const T* __restrict__ bias_r, const T* __restrict__ bias_i,
+                                    const T* __restrict__ lam, const int* __restrict__ cu_tokens, int n_seqs, int width,
+                                    int bw, float decay) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    const int g = blockIdx.y;
+    int seq, begin, end;
+    if (!scan_chunk(cu_tokens, n_seqs, g, seq, begin, end)) return;
+    if (blockIdx.x == 0)
+        for (int t = begin + threadIdx.x; t < end; t += blockDim.x) token_chunk[t] = g;
+    if (c >= width) return;
+    const int blk = c / bw, j = c - blk * bw;
+    const long long zr_at = (long long)blk * 2 * bw + j, zi_at = zr_at + bw;
+    const float br = ld(bias_r + c), bi = ld(bias_i + c);
+    const float l = ld(lam + c);
+    const float sp = fmaxf(l, 0.f) + log1pf(expf(-fabsf(l)));
+    float L = 0.f, A = 1.f;
+    for (int t = begin; t < end; ++t) {
+        const float r = 1.0f / (1.0f + expf(-(z[(long long)t * 2 * width + zr_at] + br)));
+        const float gi = 1.0f / (1.0f + expf(-(z[(long long)t * 2 * width + zi_at] + bi)));
+        const float log_a = -decay * r * sp;
+        const float a = expf(log_a);
+        const float m = sqrtf(-expm1f(2.0f * log_a));
+        L = fmaf(a, L, m * gi * u[(long long)t * width + c]);
+        A *= a;
+        loc[(long long)t * width + c] = L;
+        cum[(long long)t * width + c] = A;
+    }
+    chunk_a[(long long)g * width + c] = A;
+    chunk_l[(long long)g * width + c] = L;
+}
+
+template <typename T>
+__global__ void rglru_carry_kernel(float* __restrict__ chunk_in, float* __restrict__ state, const float* __restrict__ chunk_a,
+                                   const float* __restrict__ chunk_l, const T* __restrict__ x,
+                                   const int* __restrict__ cu_tokens, const int* __restrict__ state_slots, int width, int k,
+                                   long long x_ld, int x_off) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= width) return;
+    const int seq = blockIdx.y;
+    int g = 0;
+    for (int s = 0; s < seq; ++s) g += (cu_tokens[s + 1] - cu_tokens[s] + IA_SCAN_CHUNK - 1) / IA_SCAN_CHUNK;
+    const int first = cu_tokens[seq], last = cu_tokens[seq + 1];
+    const int nc = (last - first + IA_SCAN_CHUNK - 1) / IA_SCAN_CHUNK;
+    float* row = state + (long long)state_slots[seq] * k * width + c;
+    float S = row[0];
+    for (int i = 0; i < nc; ++i) {
+        const long long at = (long long)(g + i) * width + c;
+        chunk_in[at] = S;
+        S = fmaf(chunk_a[at], S, chunk_l[at]);
+    }
+    row[0] = S;
+    const int q = last - first;
+    for (int m = 0; m < k - 1; ++m) {
+        const int src = last - (k - 1) + m;
+        float v;
+        if (src >= first) v = ld(x + (long long)src * x_ld + x_off + c);
+        else v = row[(long long)(1 + m + q) * width];
+        row[(long long)(1 + m) * width] = v;
+    }
+}
+
+template <typename T>
+__global__ void rglru_finish_kernel(T* __restrict__ out, const float* __restrict__ loc, const float* __restrict__ cum,
+                                    const float* __restrict__ chunk_in, const int* __restrict__ token_chunk,
+                                    const T* __restrict__ branch, int width, long long b_ld, int b_off, long long total) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int t = (int)(i / width), c = (int)(i - (long long)t * width);
+    const float S = fmaf(cum[i], chunk_in[(long long)token_chunk[t] * width + c], loc[i]);
+    const float bv = ld(branch + (long long)t * b_ld + b_off + c);
+    const float y = 0.5f * bv * (1.0f + tanhf(0.7978845608028654f * (bv + 0.044715f * bv * bv * bv)));
+    st(out + i, S * y);
+}
+
+// work: 2 n width + 3 chunks width floats and n ints, chunks = n / 64 + n_seqs (ia_rglru_chunked_workspace words)
+extern "C" long long ia_rglru_chunked_workspace(int n, int n_seqs, int width) {
+    const long long chunks = n / IA_SCAN_CHUNK + n_seqs;
+    return 2LL * n * width + 3LL * chunks * width + n;
+}
+
+extern "C" int ia_rglru_scan_chunked(void* out, float* state, float* work, const float* u, const float* z,
+                                     const void* bias_r, const void* bias_i, const void* lam, const void* branch,
+                                     const void* x, const int* cu_tokens, const int* state_slots, int n, int n_seqs,
+                                     int width, int bw, int k, float decay, long long b_ld, int b_off, long long x_ld,
+                                     int x_off, int dtype, hipStream_t stream) {
+    IA_CHECK(n >= 0 && n_seqs >= 0 && width > 0 && bw > 0 && width % bw == 0 && k >= 1, "rglru_scan_chunked: bad sizes");
+    IA_CHECK(b_off >= 0 && b_off + width <= b_ld && x_off >= 0 && x_off + width <= x_ld, "rglru_scan_chunked: the branches do not fit their rows");
+    if (n == 0 || n_seqs == 0) return 0;
+    const int chunks = n / IA_SCAN_CHUNK + n_seqs;
+    IA_CHECK(chunks <= 65535 && n_seqs <= 65535, "rglru_scan_chunked: %d chunks are more than a grid takes", chunks);
+    float* loc = work;
+    float* cum = loc + (long long)n * width;
+    float* chunk_a = cum + (long long)n * width;
+    float* chunk_l = chunk_a + (long long)chunks * width;
+    float* chunk_in = chunk_l + (long long)chunks * width;
+    int* token_chunk = (int*)(chunk_in + (long long)chunks * width);
+    const dim3 g1((width + 63) / 64, chunks), g2((width + 63) / 64, n_seqs);
+    const long long total = (long long)n * width;
+    const int g3 = (int)((total + 255) / 256);
+#define IA_RUN(T)                                                                                                       \
+    rglru_chunks_kernel<T><<<g1, 64, 0, stream>>>(loc, cum, chunk_a, chunk_l, token_chunk, u, z, (const T*)bias_r,          \
+                                                  (const T*)bias_i, (const T*)lam, cu_tokens, n_seqs, width, bw, decay);    \
+    rglru_carry_kernel<T><<<g2, 64, 0, stream>>>(chunk_in, state, chunk_a, chunk_l, (const T*)x, cu_tokens, state_slots,    \
+                                                 width, k, x_ld, x_off);                                                    \
+    rglru_finish_kernel<T><<<g3, 256, 0, stream>>>((T*)out, loc, cum, chunk_in, token_chunk, (const T*)branch, width, b_ld, \
+                                                   b_off, total)
+    if (dtype == IA_F32) { IA_RUN(float); } else { IA_RUN(bf16_t); }
+#undef IA_RUN
+    IA_LAUNCH_CHECK("rglru_scan_chunked");
     return 0;
 }

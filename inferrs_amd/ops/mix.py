@@ -146,9 +146,10 @@ def head_product(x: torch.Tensor, w: torch.Tensor, *, x_off: int = 0, x_head: Op
 
 def conv_step(x: torch.Tensor, x_off: int, width: int, taps: torch.Tensor, bias: Optional[torch.Tensor],
               state: torch.Tensor, token_seq: torch.Tensor, cu_tokens: torch.Tensor,
-              state_slots: torch.Tensor) -> torch.Tensor:
+              state_slots: torch.Tensor, rounded: bool = False):
     """The causal convolution a channel over the step's tokens: x[:, x_off : x_off + width] -> 32-bit u
-    [n, width]; inputs before a request's portion come from rows 1.. of its state row ([slots, k, width])."""
+    [n, width]; inputs before a request's portion come from rows 1.. of its state row ([slots, k, width]).
+    `rounded`: returns (u, its bfloat16 copy)."""
     _dev(x, taps, bias, state, token_seq, cu_tokens, state_slots); _f32(state, "state")
     _i32(token_seq, "token_seq"); _i32(cu_tokens, "cu_tokens"); _i32(state_slots, "state_slots")
     n, k = x.shape[0], taps.shape[1]
@@ -156,17 +157,21 @@ def conv_step(x: torch.Tensor, x_off: int, width: int, taps: torch.Tensor, bias:
             or tuple(state.shape[1:]) != (k, width) or (bias is not None and (bias.numel() != width or bias.dtype != x.dtype))):
         raise KernelError(f"conv_step: taps {tuple(taps.shape)} / state {tuple(state.shape)} do not fit width {width}")
     u = torch.empty((n, width), dtype=torch.float32, device=x.device)
-    _check(library().ia_conv_step(_p(u), _p(x), _p(taps), _p(bias), _p(state), _p(token_seq), _p(cu_tokens),
+    lo = torch.empty((n, width), dtype=torch.bfloat16, device=x.device) if rounded else None
+    _check(library().ia_conv_step(_p(u), _p(lo), _p(x), _p(taps), _p(bias), _p(state), _p(token_seq), _p(cu_tokens),
                                   _p(state_slots), n, width, k, x.shape[1], x_off, _dt(x), _stream()))
-    return u
+    return (u, lo) if rounded else u
 
 
 def rglru_scan(u: torch.Tensor, z: torch.Tensor, proj: torch.Tensor, *, branch_off: int, x_off: int,
                bias_r: torch.Tensor, bias_i: torch.Tensor, lam: torch.Tensor, state: torch.Tensor,
-               cu_tokens: torch.Tensor, state_slots: torch.Tensor, block_width: int, decay: float) -> torch.Tensor:
+               cu_tokens: torch.Tensor, state_slots: torch.Tensor, block_width: int, decay: float,
+               chunked: bool = False) -> torch.Tensor:
     """The recurrence over each request's tokens, from and into its state row; returns S_t * gelu_tanh(branch_t)
     in the precision of `proj` ([n, ...]: the gelu branch at `branch_off`, the convolution's input at `x_off`).
-    z [n, 2 * width]: the gates' products before bias and sigmoid, block by block [recurrence gate | input gate]."""
+    z [n, 2 * width]: the gates' products before bias and sigmoid, block by block [recurrence gate | input gate].
+    `chunked`: chunks of 64 tokens side by side and a short walk over the chunks (steps with long portions; the
+    result differs from the token-by-token walk by rounding only)."""
     _dev(u, z, proj, bias_r, bias_i, lam, state, cu_tokens, state_slots)
     _f32(u, "u"); _f32(z, "z"); _f32(state, "state"); _i32(cu_tokens, "cu_tokens"); _i32(state_slots, "state_slots")
     n, width = u.shape
@@ -178,6 +183,14 @@ def rglru_scan(u: torch.Tensor, z: torch.Tensor, proj: torch.Tensor, *, branch_o
             raise KernelError("rglru_scan: biases and decay parameters are one entry a channel in the projections' precision")
     n_seqs = state_slots.numel()
     out = torch.empty((n, width), dtype=proj.dtype, device=proj.device)
+    if chunked:
+        lib = library()
+        work = torch.empty((lib.ia_rglru_chunked_workspace(n, n_seqs, width),), dtype=torch.float32, device=proj.device)
+        _check(lib.ia_rglru_scan_chunked(
+            _p(out), _p(state), _p(work), _p(u), _p(z), _p(bias_r), _p(bias_i), _p(lam), _p(proj), _p(proj), _p(cu_tokens),
+            _p(state_slots), n, n_seqs, width, block_width, k, ctypes.c_float(decay), proj.shape[1], branch_off,
+            proj.shape[1], x_off, _dt(proj), _stream()))
+        return out
     _check(library().ia_rglru_scan(
         _p(out), _p(state), _p(u), _p(z), _p(bias_r), _p(bias_i), _p(lam), _p(proj), _p(proj), _p(cu_tokens),
         _p(state_slots), n_seqs, width, block_width, k, ctypes.c_float(decay), proj.shape[1], branch_off,
@@ -189,18 +202,22 @@ def rglru_scan(u: torch.Tensor, z: torch.Tensor, proj: torch.Tensor, *, branch_o
 
 def route(h: torch.Tensor, router: torch.Tensor, top: int, scale: float, score: str = "sigmoid",
           renormalize: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Router logits in 32-bit (router [E, width] float32), the `top` experts by score for every row:
-    (experts int32 [n, top] best first, weights float32 [n, top] = score * scale)."""
-    _dev(h, router); _f32(router, "router")
+    """Router logits in 32-bit (router [E, width] in the precision of h: the product is the 32-bit path's, every
+    logit one chain of 32-bit multiply-adds whatever the operands are stored in), the `top` experts by score for
+    every row: (experts int32 [n, top] best first, weights float32 [n, top] = score * scale)."""
+    from . import gemm_tiled
+    _dev(h, router)
     n, W = h.shape
     E = router.shape[0]
-    if router.shape[1] != W or not (1 <= top <= min(E, MAX_TOP)) or E > MAX_EXPERTS or score not in SCORE_FUNCTIONS:
-        raise KernelError(f"route: router {tuple(router.shape)}, top {top}, score {score!r} (up to {MAX_EXPERTS} experts, "
-                          f"top up to {MAX_TOP}, scores {sorted(SCORE_FUNCTIONS)})")
+    if (router.shape[1] != W or router.dtype != h.dtype or not (1 <= top <= min(E, MAX_TOP)) or E > MAX_EXPERTS
+            or score not in SCORE_FUNCTIONS):
+        raise KernelError(f"route: router {tuple(router.shape)} {router.dtype}, top {top}, score {score!r} (up to {MAX_EXPERTS} "
+                          f"experts, top up to {MAX_TOP}, scores {sorted(SCORE_FUNCTIONS)})")
+    logits = gemm_tiled(h, router, torch.float32)
     sel = torch.empty((n, top), dtype=torch.int32, device=h.device)
     weight = torch.empty((n, top), dtype=torch.float32, device=h.device)
-    _check(library().ia_route(_p(sel), _p(weight), _p(h), _p(router), n, W, E, top, ctypes.c_float(scale),
-                              SCORE_FUNCTIONS[score], int(renormalize), _dt(h), _stream()))
+    _check(library().ia_route(_p(sel), _p(weight), _p(logits), n, E, top, ctypes.c_float(scale),
+                              SCORE_FUNCTIONS[score], int(renormalize), _stream()))
     return sel, weight
 
 

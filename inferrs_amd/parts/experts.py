@@ -53,8 +53,8 @@ class RoutedExperts(FeedForward):
         if spec.score not in ops.mix.SCORE_FUNCTIONS:
             raise SpecError(f"routed_experts: score {spec.score!r} has no kernel (known: {sorted(ops.mix.SCORE_FUNCTIONS)})")
         self.spec = spec
-        # the router stays 32-bit whatever the products are computed in
-        self.router = tensors["router"].to(device=device, dtype=torch.float32).contiguous()
+        # the router's logits are 32-bit sums whatever its matrix is stored in (`ops.route`)
+        self.router = to_compute(tensors["router"], dtype, device)
         E = spec.experts
         self.gate_up = torch.stack([torch.cat([to_compute(tensors[f"e{e}.gate"], dtype, device),
                                                to_compute(tensors[f"e{e}.up"], dtype, device)], dim=0) for e in range(E)]).contiguous()

@@ -24,6 +24,7 @@ from .linear import Linear, to_compute
 @register_mixer("rglru")
 class GatedRecurrence(Mixer):
     graph_safe = True
+    CHUNKED_FROM = 64              # steps whose longest portion has more tokens walk it in chunks side by side
 
     @classmethod
     def tensors(cls, spec: GatedRecurrenceSpec) -> Dict[str, TensorSpec]:
@@ -62,9 +63,12 @@ class GatedRecurrence(Mixer):
         s = self.spec
         w, bw = s.width, s.width // s.blocks
         proj = self.proj(h)                                      # [n, gelu branch | convolution's input]
-        u = ops.conv_step(proj, w, w, self.taps, self.conv_bias, cache.state, ctx.token_seq, ctx.cu_tokens, ctx.state_slots)
-        z = ops.head_product(u, self.gates, out_dtype=torch.float32)                  # [n, blocks * 2 bw]
+        lo = proj.dtype == torch.bfloat16               # the gates' products take u in the projections' precision
+        u = ops.conv_step(proj, w, w, self.taps, self.conv_bias, cache.state, ctx.token_seq, ctx.cu_tokens, ctx.state_slots,
+                          rounded=lo)
+        u, u_in = u if lo else (u, u)
+        z = ops.head_product(u_in, self.gates, out_dtype=torch.float32)               # [n, blocks * 2 bw]
         mixed = ops.rglru_scan(u, z, proj, branch_off=0, x_off=w, bias_r=self.bias_r, bias_i=self.bias_i, lam=self.lam,
                                state=cache.state, cu_tokens=ctx.cu_tokens, state_slots=ctx.state_slots, block_width=bw,
-                               decay=s.decay)
+                               decay=s.decay, chunked=ctx.max_q_len > self.CHUNKED_FROM)
         return self.o(mixed)

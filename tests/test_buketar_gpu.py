@@ -118,8 +118,9 @@ def plain_recurrence_pieces(proj, w, width):
     return u, torch.stack(rows) * y
 
 
+@pytest.mark.parametrize("chunked", [False, True])
 @pytest.mark.parametrize("width, blocks, taps", [(40, 2, 4), (48, 1, 1), (96, 3, 2), (130, 5, 7)])
-def test_recurrence_carried_over_portions(width, blocks, taps):
+def test_recurrence_carried_over_portions(width, blocks, taps, chunked):
     """Two requests in slots 3 and 1 of a dirty state array that is cleared for them, fed in portions of unequal
     sizes side by side (down to one token, shorter than the convolution); the result is that of each alone and whole."""
     from inferrs_amd import ops
@@ -129,13 +130,13 @@ def test_recurrence_carried_over_portions(width, blocks, taps):
          "ra": torch.randn(blocks, bw, bw, generator=g) / bw ** 0.5, "ra.b": 0.3 * torch.randn(blocks, bw, generator=g),
          "ri": torch.randn(blocks, bw, bw, generator=g) / bw ** 0.5, "ri.b": 0.3 * torch.randn(blocks, bw, generator=g),
          "lam": torch.empty(width).uniform_(-8.0, 1.0, generator=g)}
-    lens = {3: 131, 1: 58}
+    lens = {3: 331, 1: 58}
     proj = {s: torch.randn(n, 2 * width, generator=g) for s, n in lens.items()}
     want = {s: plain_recurrence_pieces(proj[s].double(), {k: v.double() for k, v in w.items()}, width) for s in lens}
     state = torch.full((5, taps, width), 7.0, device="cuda")
     state[3].zero_(); state[1].zero_()
     gates = dev(torch.cat([w["ra"], w["ri"]], dim=1))
-    cuts = {3: [1, 2, 64, 1, 3, 33, 27], 1: [5, 1, 1, 2, 40, 9]}
+    cuts = {3: [1, 2, 64, 1, 3, 33, 27, 200], 1: [5, 1, 1, 2, 40, 9]}
     at = {s: 0 for s in lens}
     got_u = {s: [] for s in lens}
     got = {s: [] for s in lens}
@@ -149,9 +150,10 @@ def test_recurrence_carried_over_portions(width, blocks, taps):
         seq = dev(torch.tensor([i for i, c in enumerate(counts) for _ in range(c)], dtype=torch.int32))
         slots = dev(torch.tensor(live, dtype=torch.int32))
         u = ops.conv_step(rows, width, width, dev(w["conv"]), dev(w["conv.b"]), state, seq, cu, slots)
+        assert ops.conv_step(rows, width, width, dev(w["conv"]), dev(w["conv.b"]), state, seq, cu, slots, rounded=True)[1].dtype == torch.bfloat16
         z = ops.head_product(u, gates, out_dtype=torch.float32)
         out = ops.rglru_scan(u, z, rows, branch_off=0, x_off=width, bias_r=dev(w["ra.b"].reshape(-1)), bias_i=dev(w["ri.b"].reshape(-1)),
-                             lam=dev(w["lam"]), state=state, cu_tokens=cu, state_slots=slots, block_width=bw, decay=8.0)
+                             lam=dev(w["lam"]), state=state, cu_tokens=cu, state_slots=slots, block_width=bw, decay=8.0, chunked=chunked)
         o = 0
         for s, c in zip(live, counts):
             got_u[s].append(u[o:o + c].cpu()); got[s].append(out[o:o + c].cpu())
