@@ -173,18 +173,21 @@ int ia_rglru_scan_chunked(void* out, float* state, float* work, const float* u, 
                           int x_off, int dtype, hipStream_t stream);
 
 // ---- routed experts (experts.hip) --------------------------------------------------------------------------------
-// score_fn: 0 sigmoid, 1 softmax over all experts
-int ia_route(int* sel, float* weight, const float* logits, int n, int E, int top, float scale, int score_fn,
-             int renorm, hipStream_t stream);
+// score_fn: 0 sigmoid, 1 softmax over all experts.  tile: rows of a row tile, 32, 64 or 128 (the plan, gate_up and down
+// of one call agree).  tiled: the weights are stored as tiles of 64 features x 64 k values, zero-padded: w_gu
+// [E][2][ceil(ff / 64)][ceil(W / 64)][64][64], w_down [E][ceil(W / 64)][ceil(ff / 64)][64][64] (bfloat16, matrix cores);
+// else w_gu [E][2 ff][W], w_down [E][W][ff].
+int ia_route(int* sel, float* weight, const void* h, const void* router, int n, int W, int E, int top,
+             float scale, int score_fn, int renorm, int dtype, hipStream_t stream);
 int ia_route_tiles(int pairs, int E);
 int ia_route_plan(int* order, int* tile_expert, int* tile_first, int* tile_rows, int* meta, const int* sel,
-                  int pairs, int E, hipStream_t stream);
+                  int pairs, int E, int tile, hipStream_t stream);
 int ia_experts_gate_up(void* act, const void* h, const void* w_gu, const int* order, const int* tile_expert,
                        const int* tile_first, const int* tile_rows, const int* meta, int pairs, int E, int top,
-                       int W, int ff, float limit, float alpha, int dtype, hipStream_t stream);
+                       int W, int ff, float limit, float alpha, int tile, int tiled, int dtype, hipStream_t stream);
 int ia_experts_down(float* y, const void* act, const void* w_down, const int* order, const int* tile_expert,
                     const int* tile_first, const int* tile_rows, const int* meta, int pairs, int E, int W,
-                    int ff, int dtype, hipStream_t stream);
+                    int ff, int tile, int tiled, int dtype, hipStream_t stream);
 
 // Built per head size (-DIA_HEAD_DIM) into a library of its own.
 int ia_attention_mfma_head_dim(void);

@@ -1,8 +1,8 @@
 // Routed experts: a router scores every expert for a token, the `top` best are run and their outputs added up
 // with the scores as weights.
 //
-//   route      a wave a token, from the router's 32-bit logits (a product of the 32-bit path): scores = sigmoid (or
-//              softmax), the top experts by score (ties: the lower index), weights = score * scale (optionally
+//   route      a wave a token: router logits as 32-bit sums whatever row and matrix are stored in, scores = sigmoid
+//              (or softmax), the top experts by score (ties: the lower index), weights = score * scale (optionally
 //              renormalised over the chosen).
 //   plan       one block: the (token, k) pairs ordered by expert, and a table of row tiles (expert, first pair, rows),
 //              all on the device: the host never learns how many tokens an expert got.
@@ -19,15 +19,70 @@
 
 enum { IA_SCORE_SIGMOID = 0, IA_SCORE_SOFTMAX = 1 };
 
+// eight neighbouring values of a row as 32-bit floats
+__device__ __forceinline__ void load8(const float* p, float (&v)[8]) {
+    const float4 a = *reinterpret_cast<const float4*>(p), b = *reinterpret_cast<const float4*>(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+__device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
+    const uint4 a = *reinterpret_cast<const uint4*>(p);
+    const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __uint_as_float(w[i] << 16);
+        v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+}
+
+#define IA_ROUTE_GROUP 32      // experts whose sums a wave holds at a time
+
+// The logits: a lane owns the features 8 lane + 512 i of the row and adds its products up in that order (32-bit
+// multiply-adds), then the lanes' sums meet in a butterfly: an order that depends on the width alone.  VEC: the width
+// is a multiple of 8 (16-byte loads); else element by element.
+template <typename T, bool VEC>
 __global__ __launch_bounds__(64) void route_kernel(int* __restrict__ sel, float* __restrict__ weight,
-                                                   const float* __restrict__ logits, int n, int E, int top, float scale,
-                                                   int score_fn, int renorm) {
+                                                   const T* __restrict__ h, const T* __restrict__ wr, int n, int W, int E,
+                                                   int top, float scale, int score_fn, int renorm) {
     const int t = blockIdx.x, lane = threadIdx.x;
+    const T* row = h + (long long)t * W;
     float z[IA_MAX_EXPERTS / IA_WAVE];             // expert e lives in lane e % 64, register e / 64
 #pragma unroll
-    for (int q = 0; q < IA_MAX_EXPERTS / IA_WAVE; ++q) {
-        const int e = q * IA_WAVE + lane;
-        z[q] = e < E ? logits[(long long)t * E + e] : -INFINITY;
+    for (int q = 0; q < IA_MAX_EXPERTS / IA_WAVE; ++q) z[q] = -INFINITY;
+    for (int e0 = 0; e0 < E; e0 += IA_ROUTE_GROUP) {
+        float acc[IA_ROUTE_GROUP];
+#pragma unroll
+        for (int j = 0; j < IA_ROUTE_GROUP; ++j) acc[j] = 0.f;
+        for (int c0 = lane * 8; c0 < W; c0 += IA_WAVE * 8) {
+            float x[8];
+            if (VEC) {
+                load8(row + c0, x);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 8; ++i) x[i] = c0 + i < W ? ld(row + c0 + i) : 0.f;
+            }
+#pragma unroll
+            for (int j = 0; j < IA_ROUTE_GROUP; ++j) {
+                // (an expert beyond the last reads the last one's row: no branch stands between the loads)
+                const T* w = wr + (long long)(e0 + j < E ? e0 + j : E - 1) * W + c0;
+                float wv[8];
+                if (VEC) {
+                    load8(w, wv);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) wv[i] = c0 + i < W ? ld(w + i) : 0.f;
+                }
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[j] = fmaf(x[i], wv[i], acc[j]);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < IA_ROUTE_GROUP; ++j) {
+            const float total = wave_sum(acc[j]);
+            const int e = e0 + j;
+#pragma unroll
+            for (int q = 0; q < IA_MAX_EXPERTS / IA_WAVE; ++q)
+                if (e < E && e == q * IA_WAVE + lane) z[q] = total;
+        }
     }
     float zmax = -INFINITY, denom = 1.f;
     if (score_fn == IA_SCORE_SOFTMAX) {
@@ -71,7 +126,7 @@ __global__ __launch_bounds__(64) void route_kernel(int* __restrict__ sel, float*
 __global__ __launch_bounds__(1024) void route_plan_kernel(int* __restrict__ order, int* __restrict__ tile_expert,
                                                           int* __restrict__ tile_first, int* __restrict__ tile_rows,
                                                           int* __restrict__ meta, const int* __restrict__ sel, int pairs,
-                                                          int E) {
+                                                          int E, int tile) {
     __shared__ int count[IA_MAX_EXPERTS], first[IA_MAX_EXPERTS], tile0[IA_MAX_EXPERTS], cursor[IA_MAX_EXPERTS];
     for (int e = threadIdx.x; e < E; e += blockDim.x) count[e] = cursor[e] = 0;
     __syncthreads();
@@ -83,17 +138,17 @@ __global__ __launch_bounds__(1024) void route_plan_kernel(int* __restrict__ orde
             first[e] = at;
             tile0[e] = tiles;
             at += count[e];
-            tiles += (count[e] + IA_TM - 1) / IA_TM;
+            tiles += (count[e] + tile - 1) / tile;
         }
         meta[0] = tiles;
     }
     __syncthreads();
     for (int e = threadIdx.x; e < E; e += blockDim.x) {
-        const int tiles = (count[e] + IA_TM - 1) / IA_TM;
+        const int tiles = (count[e] + tile - 1) / tile;
         for (int i = 0; i < tiles; ++i) {
             tile_expert[tile0[e] + i] = e;
-            tile_first[tile0[e] + i] = first[e] + i * IA_TM;
-            tile_rows[tile0[e] + i] = min(IA_TM, count[e] - i * IA_TM);
+            tile_first[tile0[e] + i] = first[e] + i * tile;
+            tile_rows[tile0[e] + i] = min(tile, count[e] - i * tile);
         }
     }
     for (int p = threadIdx.x; p < pairs; p += blockDim.x) {
@@ -165,7 +220,9 @@ __global__ __launch_bounds__(256) void experts_down_kernel(float* __restrict__ y
     }
 }
 
-// The same two products on the matrix cores (bfloat16; widths in steps of 8).
+// The same two products on the matrix cores (bfloat16; widths in steps of 8) over weights stored as tiles (see
+// tile_mfma.h): w_gu [E][2][ceil(ff / 64)][ceil(W / 64)][64][64], w_down [E][ceil(W / 64)][ceil(ff / 64)][64][64].
+template <int RT, int FT>
 __global__ __launch_bounds__(256) void experts_gate_up_mfma_kernel(bf16_t* __restrict__ act, const bf16_t* __restrict__ h,
                                                                    const bf16_t* __restrict__ w_gu,
                                                                    const int* __restrict__ order,
@@ -174,29 +231,37 @@ __global__ __launch_bounds__(256) void experts_gate_up_mfma_kernel(bf16_t* __res
                                                                    const int* __restrict__ tile_rows,
                                                                    const int* __restrict__ meta, int top, int W, int ff,
                                                                    float limit, float alpha) {
-    __shared__ TileSharedMfma sh;
+    using Tile = TileMfma<RT, FT, 64, true>;
+    __shared__ typename Tile::Shared sh;
     const int tile = blockIdx.y;
     if (tile >= meta[0]) return;
-    const int e = tile_expert[tile], first = tile_first[tile], rows = tile_rows[tile], col0 = blockIdx.x * IA_MN;
-    tm_f32x4 g[2], u[2];
+    const int e = tile_expert[tile], first = tile_first[tile], rows = tile_rows[tile], col0 = blockIdx.x * Tile::FEATURES;
+    const int fbs = (ff + 63) / 64, chunks = (W + 63) / 64;
+    tm_f32x4 g[FT][RT], u[FT][RT];
     auto xrow = [&](int i) -> const bf16_t* { return i < rows ? h + (long long)(order[first + i] / top) * W : nullptr; };
-    const bf16_t* wg = w_gu + ((long long)e * 2 * ff + col0) * W;
-    tile_product_mfma<true>(g, u, sh, xrow, wg, wg + (long long)ff * W, ff - col0, W, W);
+    const long long matrix = (long long)fbs * chunks * 4096;
+    const bf16_t* wg = w_gu + (long long)e * 2 * matrix + (long long)(col0 / 64) * chunks * 4096;
+    Tile::product_tiled(g, u, sh, xrow, wg, wg + matrix, fbs - col0 / 64, chunks, W);
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
 #pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
+    for (int rt = 0; rt < RT; ++rt) {
         const int i = 16 * rt + (lane & 15);
-        if (i >= rows) continue;
 #pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int j = col0 + 16 * wave + 4 * (lane >> 4) + q;
-            if (j >= ff) continue;
-            const float gv = fminf(g[rt][q], limit), uv = fminf(fmaxf(u[rt][q], -limit), limit);
-            st(act + (long long)(first + i) * ff + j, gv / (1.0f + expf(-alpha * gv)) * (uv + 1.0f));
+        for (int ft = 0; ft < FT; ++ft) {
+            const int j0 = col0 + 16 * (wave * FT + ft) + 4 * (lane >> 4);
+            const tm_f32x4 gq = g[ft][rt], uq = u[ft][rt];
+            const float gs[4] = {gq[0], gq[1], gq[2], gq[3]}, us[4] = {uq[0], uq[1], uq[2], uq[3]};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                if (i >= rows || j0 + q >= ff) continue;
+                const float gv = fminf(gs[q], limit), uv = fminf(fmaxf(us[q], -limit), limit);
+                st(act + (long long)(first + i) * ff + j0 + q, gv / (1.0f + expf(-alpha * gv)) * (uv + 1.0f));
+            }
         }
     }
 }
 
+template <int RT, int FT>
 __global__ __launch_bounds__(256) void experts_down_mfma_kernel(float* __restrict__ y, const bf16_t* __restrict__ act,
                                                                 const bf16_t* __restrict__ w_down,
                                                                 const int* __restrict__ order,
@@ -204,60 +269,71 @@ __global__ __launch_bounds__(256) void experts_down_mfma_kernel(float* __restric
                                                                 const int* __restrict__ tile_first,
                                                                 const int* __restrict__ tile_rows,
                                                                 const int* __restrict__ meta, int W, int ff) {
-    __shared__ TileSharedMfma sh;
+    using Tile = TileMfma<RT, FT, 64, false>;
+    __shared__ typename Tile::Shared sh;
     const int tile = blockIdx.y;
     if (tile >= meta[0]) return;
-    const int e = tile_expert[tile], first = tile_first[tile], rows = tile_rows[tile], col0 = blockIdx.x * IA_MN;
-    tm_f32x4 acc[2], unused[2];
+    const int e = tile_expert[tile], first = tile_first[tile], rows = tile_rows[tile], col0 = blockIdx.x * Tile::FEATURES;
+    const int fbs = (W + 63) / 64, chunks = (ff + 63) / 64;
+    tm_f32x4 acc[FT][RT], unused[FT][RT];
     auto xrow = [&](int i) -> const bf16_t* { return i < rows ? act + (long long)(first + i) * ff : nullptr; };
-    const bf16_t* wd = w_down + ((long long)e * W + col0) * ff;
-    tile_product_mfma<false>(acc, unused, sh, xrow, wd, wd, W - col0, ff, ff);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-#pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
-        const int i = 16 * rt + (lane & 15);
-        if (i >= rows) continue;
-        const long long pair = order[first + i];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int c = col0 + 16 * wave + 4 * (lane >> 4) + q;
-            if (c < W) y[pair * W + c] = acc[rt][q];
-        }
-    }
+    const bf16_t* wd = w_down + ((long long)e * fbs + col0 / 64) * chunks * 4096;
+    Tile::product_tiled(acc, unused, sh, xrow, wd, wd, fbs - col0 / 64, chunks, ff);
+    Tile::each([&](int i, int f, int ft, int rt, int q) {
+        const int c = col0 + f;
+        if (i < rows && c < W) y[(long long)order[first + i] * W + c] = acc[ft][rt][q];
+    });
 }
 
-extern "C" int ia_route(int* sel, float* weight, const float* logits, int n, int E, int top, float scale, int score_fn,
-                        int renorm, hipStream_t stream) {
-    IA_CHECK(n >= 0 && E >= 1 && E <= IA_MAX_EXPERTS && top >= 1 && top <= E && top <= IA_MAX_TOP,
-             "route: n=%d experts=%d (up to %d) top=%d (up to %d)", n, E, IA_MAX_EXPERTS, top, IA_MAX_TOP);
+extern "C" int ia_route(int* sel, float* weight, const void* h, const void* router, int n, int W, int E, int top,
+                        float scale, int score_fn, int renorm, int dtype, hipStream_t stream) {
+    IA_CHECK(n >= 0 && W > 0 && E >= 1 && E <= IA_MAX_EXPERTS && top >= 1 && top <= E && top <= IA_MAX_TOP,
+             "route: n=%d width=%d experts=%d (up to %d) top=%d (up to %d)", n, W, E, IA_MAX_EXPERTS, top, IA_MAX_TOP);
     IA_CHECK(score_fn == IA_SCORE_SIGMOID || score_fn == IA_SCORE_SOFTMAX, "route: unknown score function %d", score_fn);
     if (n == 0) return 0;
-    route_kernel<<<n, 64, 0, stream>>>(sel, weight, logits, n, E, top, scale, score_fn, renorm);
+    const bool vec = W % 8 == 0 && tile_mfma_aligned(h) && tile_mfma_aligned(router);
+#define IA_ROUTE(T, V) route_kernel<T, V><<<n, 64, 0, stream>>>(sel, weight, (const T*)h, (const T*)router, n, W, E, top, scale, score_fn, renorm)
+    if (dtype == IA_F32) { if (vec) IA_ROUTE(float, true); else IA_ROUTE(float, false); }
+    else { if (vec) IA_ROUTE(bf16_t, true); else IA_ROUTE(bf16_t, false); }
+#undef IA_ROUTE
     IA_LAUNCH_CHECK("route");
     return 0;
 }
 
-// The most tiles that `pairs` pairs over E experts can make: the grids of the two products.
-extern "C" int ia_route_tiles(int pairs, int E) { return (pairs + IA_TM - 1) / IA_TM + (E < pairs ? E : pairs); }
+// The most tiles of `tile` rows that `pairs` pairs over E experts can make: the grids of the two products.
+static int route_tiles(int pairs, int E, int tile) { return (pairs + tile - 1) / tile + (E < pairs ? E : pairs); }
+extern "C" int ia_route_tiles(int pairs, int E) { return route_tiles(pairs, E, IA_TM); }
 
+// tile: rows of a tile, 32 (every kernel) or 64 or 128 (the matrix cores' large shapes, for many rows an expert)
 extern "C" int ia_route_plan(int* order, int* tile_expert, int* tile_first, int* tile_rows, int* meta, const int* sel,
-                             int pairs, int E, hipStream_t stream) {
-    IA_CHECK(pairs >= 0 && E >= 1 && E <= IA_MAX_EXPERTS, "route_plan: pairs=%d experts=%d", pairs, E);
-    route_plan_kernel<<<1, 1024, 0, stream>>>(order, tile_expert, tile_first, tile_rows, meta, sel, pairs, E);
+                             int pairs, int E, int tile, hipStream_t stream) {
+    IA_CHECK(pairs >= 0 && E >= 1 && E <= IA_MAX_EXPERTS && (tile == 32 || tile == 64 || tile == 128), "route_plan: pairs=%d experts=%d tile=%d",
+             pairs, E, tile);
+    route_plan_kernel<<<1, 1024, 0, stream>>>(order, tile_expert, tile_first, tile_rows, meta, sel, pairs, E, tile);
     IA_LAUNCH_CHECK("route_plan");
     return 0;
 }
 
 extern "C" int ia_experts_gate_up(void* act, const void* h, const void* w_gu, const int* order, const int* tile_expert,
                                   const int* tile_first, const int* tile_rows, const int* meta, int pairs, int E, int top,
-                                  int W, int ff, float limit, float alpha, int dtype, hipStream_t stream) {
-    IA_CHECK(pairs >= 0 && W > 0 && ff > 0 && top >= 1 && limit > 0.f, "experts_gate_up: bad sizes");
+                                  int W, int ff, float limit, float alpha, int tile, int tiled, int dtype, hipStream_t stream) {
+    IA_CHECK(pairs >= 0 && W > 0 && ff > 0 && top >= 1 && limit > 0.f && (tile == 32 || tile == 64 || tile == 128), "experts_gate_up: bad sizes");
     if (pairs == 0) return 0;
-    const dim3 grid((ff + IA_TN - 1) / IA_TN, ia_route_tiles(pairs, E));
+    IA_CHECK(!tiled || (dtype == IA_BF16 && W % 8 == 0 && tile_mfma_aligned(h) && tile_mfma_aligned(w_gu)),
+             "experts_gate_up: weights stored as tiles are the matrix cores' (bfloat16, widths in steps of 8)");
+    IA_CHECK(tile == 32 || tiled, "experts_gate_up: tiles of 64 or 128 rows go with weights stored as tiles");
+    const int features = tile == 32 ? 64 : 128;
+    const dim3 grid((ff + features - 1) / features, route_tiles(pairs, E, tile));
     IA_CHECK(grid.y <= 65535, "experts_gate_up: %u row tiles are more than a grid takes", grid.y);
-    if (dtype == IA_BF16 && W % 8 == 0 && tile_mfma_aligned(h) && tile_mfma_aligned(w_gu))
-        experts_gate_up_mfma_kernel<<<grid, 256, 0, stream>>>((bf16_t*)act, (const bf16_t*)h, (const bf16_t*)w_gu, order, tile_expert,
-                                                              tile_first, tile_rows, meta, top, W, ff, limit, alpha);
+    if (tiled && tile == 128)
+        experts_gate_up_mfma_kernel<8, 2><<<grid, 256, 0, stream>>>((bf16_t*)act, (const bf16_t*)h, (const bf16_t*)w_gu, order,
+                                                                    tile_expert, tile_first, tile_rows, meta, top, W, ff, limit, alpha);
+    else if (tiled && tile == 64)
+        experts_gate_up_mfma_kernel<4, 2><<<grid, 256, 0, stream>>>((bf16_t*)act, (const bf16_t*)h, (const bf16_t*)w_gu, order,
+                                                                    tile_expert, tile_first, tile_rows, meta, top, W, ff, limit, alpha);
+    else if (tiled)
+        experts_gate_up_mfma_kernel<2, 1><<<grid, 256, 0, stream>>>((bf16_t*)act, (const bf16_t*)h, (const bf16_t*)w_gu, order,
+                                                                    tile_expert, tile_first, tile_rows, meta, top, W, ff, limit, alpha);
     else if (dtype == IA_F32)
         experts_gate_up_kernel<float><<<grid, 256, 0, stream>>>((float*)act, (const float*)h, (const float*)w_gu, order,
                                                                 tile_expert, tile_first, tile_rows, meta, top, W, ff, limit, alpha);
@@ -270,14 +346,24 @@ extern "C" int ia_experts_gate_up(void* act, const void* h, const void* w_gu, co
 
 extern "C" int ia_experts_down(float* y, const void* act, const void* w_down, const int* order, const int* tile_expert,
                                const int* tile_first, const int* tile_rows, const int* meta, int pairs, int E, int W,
-                               int ff, int dtype, hipStream_t stream) {
-    IA_CHECK(pairs >= 0 && W > 0 && ff > 0, "experts_down: bad sizes");
+                               int ff, int tile, int tiled, int dtype, hipStream_t stream) {
+    IA_CHECK(pairs >= 0 && W > 0 && ff > 0 && (tile == 32 || tile == 64 || tile == 128), "experts_down: bad sizes");
     if (pairs == 0) return 0;
-    const dim3 grid((W + IA_TN - 1) / IA_TN, ia_route_tiles(pairs, E));
+    IA_CHECK(!tiled || (dtype == IA_BF16 && ff % 8 == 0 && tile_mfma_aligned(act) && tile_mfma_aligned(w_down)),
+             "experts_down: weights stored as tiles are the matrix cores' (bfloat16, widths in steps of 8)");
+    IA_CHECK(tile == 32 || tiled, "experts_down: tiles of 64 or 128 rows go with weights stored as tiles");
+    const int features = tile == 32 ? 64 : 128;
+    const dim3 grid((W + features - 1) / features, route_tiles(pairs, E, tile));
     IA_CHECK(grid.y <= 65535, "experts_down: %u row tiles are more than a grid takes", grid.y);
-    if (dtype == IA_BF16 && ff % 8 == 0 && tile_mfma_aligned(act) && tile_mfma_aligned(w_down))
-        experts_down_mfma_kernel<<<grid, 256, 0, stream>>>(y, (const bf16_t*)act, (const bf16_t*)w_down, order, tile_expert, tile_first,
-                                                           tile_rows, meta, W, ff);
+    if (tiled && tile == 128)
+        experts_down_mfma_kernel<8, 2><<<grid, 256, 0, stream>>>(y, (const bf16_t*)act, (const bf16_t*)w_down, order, tile_expert,
+                                                                 tile_first, tile_rows, meta, W, ff);
+    else if (tiled && tile == 64)
+        experts_down_mfma_kernel<4, 2><<<grid, 256, 0, stream>>>(y, (const bf16_t*)act, (const bf16_t*)w_down, order, tile_expert,
+                                                                 tile_first, tile_rows, meta, W, ff);
+    else if (tiled)
+        experts_down_mfma_kernel<2, 1><<<grid, 256, 0, stream>>>(y, (const bf16_t*)act, (const bf16_t*)w_down, order, tile_expert,
+                                                                 tile_first, tile_rows, meta, W, ff);
     else if (dtype == IA_F32)
         experts_down_kernel<float><<<grid, 256, 0, stream>>>(y, (const float*)act, (const float*)w_down, order, tile_expert,
                                                              tile_first, tile_rows, meta, W, ff);

@@ -137,35 +137,29 @@ __global__ __launch_bounds__(256) void head_product_kernel(
 }
 
 // The same on the matrix cores: bfloat16 rows and matrices, k_in and every offset a multiple of 8.
-template <typename TO>
+template <typename TO, int RT, int FT, int KC>
 __global__ __launch_bounds__(256) void head_product_mfma_kernel(
     TO* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, const bf16_t* __restrict__ gate, int n,
     int n_out, int k_in, long long x_ld, int x_off, int x_head, long long o_ld, int o_off, int o_head, long long g_ld,
     int g_off) {
-    __shared__ TileSharedMfma sh;
-    const int h = blockIdx.z, row0 = blockIdx.y * IA_MM, col0 = blockIdx.x * IA_MN;
-    tm_f32x4 acc[2], unused[2];
+    using Tile = TileMfma<RT, FT, KC, false>;
+    __shared__ typename Tile::Shared sh;
+    const int h = blockIdx.z, row0 = blockIdx.y * Tile::ROWS, col0 = blockIdx.x * Tile::FEATURES;
+    tm_f32x4 acc[FT][RT], unused[FT][RT];
     const bf16_t* xb = x + x_off + (long long)h * x_head;
     auto xrow = [&](int i) -> const bf16_t* { return row0 + i < n ? xb + (long long)(row0 + i) * x_ld : nullptr; };
     const bf16_t* wt = w + ((long long)h * n_out + col0) * k_in;
-    tile_product_mfma<false>(acc, unused, sh, xrow, wt, wt, n_out - col0, k_in, k_in);
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-#pragma unroll
-    for (int rt = 0; rt < 2; ++rt) {
-        const int t = row0 + 16 * rt + (lane & 15);
-        if (t >= n) continue;
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int j = col0 + 16 * wave + 4 * (lane >> 4) + q;
-            if (j >= n_out) continue;
-            float v = acc[rt][q];
-            if (gate != nullptr) {
-                const float g = ld(gate + (long long)t * g_ld + g_off + (long long)h * n_out + j);
-                v = v / (1.0f + expf(-g));
-            }
-            st(out + (long long)t * o_ld + o_off + (long long)h * o_head + j, v);
+    Tile::product(acc, unused, sh, xrow, wt, wt, n_out - col0, k_in, k_in);
+    Tile::each([&](int i, int f, int ft, int rt, int q) {
+        const int t = row0 + i, j = col0 + f;
+        if (t >= n || j >= n_out) return;
+        float v = acc[ft][rt][q];
+        if (gate != nullptr) {
+            const float g = ld(gate + (long long)t * g_ld + g_off + (long long)h * n_out + j);
+            v = v / (1.0f + expf(-g));
         }
-    }
+        st(out + (long long)t * o_ld + o_off + (long long)h * o_head + j, v);
+    });
 }
 
 // dtypes: 0 float32, 1 bfloat16 (x and gate share one).  Combinations built: x and w and out alike; 32-bit results of
@@ -189,14 +183,17 @@ extern "C" int ia_head_product(void* out, const void* x, const void* w, const vo
                                                               g_ld, g_off)
     const bool cores = x_dtype == IA_BF16 && w_dtype == IA_BF16 && k_in % 8 == 0 && x_ld % 8 == 0 && x_off % 8 == 0 &&
                        x_head % 8 == 0 && tile_mfma_aligned(x) && tile_mfma_aligned(w);
-    if (cores && out_dtype == IA_BF16)
-        head_product_mfma_kernel<bf16_t><<<grid, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, (const bf16_t*)w,
-                                                                   (const bf16_t*)gate, n, n_out, k_in, x_ld, x_off, x_head,
-                                                                   o_ld, o_off, o_head, g_ld, g_off);
-    else if (cores && out_dtype == IA_F32)
-        head_product_mfma_kernel<float><<<grid, 256, 0, stream>>>((float*)out, (const bf16_t*)x, (const bf16_t*)w,
-                                                                  (const bf16_t*)gate, n, n_out, k_in, x_ld, x_off, x_head,
-                                                                  o_ld, o_off, o_head, g_ld, g_off);
+    const bool large = n >= 64 && n_out >= 128;
+    const dim3 big((n_out + 127) / 128, (n + 63) / 64, H);
+    (void)big;
+#define IA_CORES(TO, RT, FT, KC, G)                                                                                            \
+    head_product_mfma_kernel<TO, RT, FT, KC><<<G, 256, 0, stream>>>((TO*)out, (const bf16_t*)x, (const bf16_t*)w,                 \
+                                                                    (const bf16_t*)gate, n, n_out, k_in, x_ld, x_off, x_head,    \
+                                                                    o_ld, o_off, o_head, g_ld, g_off)
+    if (cores && out_dtype == IA_BF16 && large) IA_CORES(bf16_t, 4, 2, 64, big);
+    else if (cores && out_dtype == IA_BF16) IA_CORES(bf16_t, 2, 1, 64, grid);
+    else if (cores && out_dtype == IA_F32 && large) IA_CORES(float, 4, 2, 64, big);
+    else if (cores && out_dtype == IA_F32) IA_CORES(float, 2, 1, 64, grid);
     else if (x_dtype == IA_F32 && w_dtype == IA_F32 && out_dtype == IA_F32) IA_LAUNCH(float, float, float);
     else if (x_dtype == IA_BF16 && w_dtype == IA_BF16 && out_dtype == IA_BF16) IA_LAUNCH(bf16_t, bf16_t, bf16_t);
     else if (x_dtype == IA_F32 && w_dtype == IA_BF16 && out_dtype == IA_F32) IA_LAUNCH(float, bf16_t, float);
@@ -206,6 +203,7 @@ extern "C" int ia_head_product(void* out, const void* x, const void* w, const vo
         return 1;
     }
 #undef IA_LAUNCH
+#undef IA_CORES
     IA_LAUNCH_CHECK("head_product");
     return 0;
 }

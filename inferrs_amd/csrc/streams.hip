@@ -36,6 +36,7 @@ __global__ __launch_bounds__(256) void streams_step_kernel(
     __syncthreads();
     float* xr = streams + (long long)row * S * W;
     float sq = 0.f;
+#pragma unroll 4
     for (int c = threadIdx.x; c < W; c += blockDim.x) {
         float x[IA_MAX_STREAMS];
 #pragma unroll

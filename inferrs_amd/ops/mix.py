@@ -4,6 +4,7 @@ Shape checks on the host, then one C call a kernel; no other implementation stan
 from __future__ import annotations
 
 import ctypes
+import os
 from typing import Optional, Tuple
 
 import torch
@@ -14,6 +15,8 @@ MAX_STREAMS = 8
 MAX_EXPERTS = 256
 MAX_TOP = 16
 ROW_TILE = 32                 # rows of a tile of the grouped products
+LARGE_TILE = int(os.environ.get("INFERRS_AMD_EXPERT_TILE", "64"))     # rows of the matrix cores' large tile: 64 or 128
+LARGE_TILE_FROM = 0.75        # rows an expert (on average), in large tiles, from which the experts' products take them
 SCORE_FUNCTIONS = {"sigmoid": 0, "softmax": 1}
 
 
@@ -202,10 +205,9 @@ def rglru_scan(u: torch.Tensor, z: torch.Tensor, proj: torch.Tensor, *, branch_o
 
 def route(h: torch.Tensor, router: torch.Tensor, top: int, scale: float, score: str = "sigmoid",
           renormalize: bool = False) -> Tuple[torch.Tensor, torch.Tensor]:
-    """Router logits in 32-bit (router [E, width] in the precision of h: the product is the 32-bit path's, every
-    logit one chain of 32-bit multiply-adds whatever the operands are stored in), the `top` experts by score for
-    every row: (experts int32 [n, top] best first, weights float32 [n, top] = score * scale)."""
-    from . import gemm_tiled
+    """Router logits in 32-bit (router [E, width] in the precision of h; every logit is a sum of 32-bit
+    multiply-adds in an order that the width alone decides), the `top` experts by score for every row:
+    (experts int32 [n, top] best first, weights float32 [n, top] = score * scale)."""
     _dev(h, router)
     n, W = h.shape
     E = router.shape[0]
@@ -213,38 +215,67 @@ def route(h: torch.Tensor, router: torch.Tensor, top: int, scale: float, score: 
             or score not in SCORE_FUNCTIONS):
         raise KernelError(f"route: router {tuple(router.shape)} {router.dtype}, top {top}, score {score!r} (up to {MAX_EXPERTS} "
                           f"experts, top up to {MAX_TOP}, scores {sorted(SCORE_FUNCTIONS)})")
-    logits = gemm_tiled(h, router, torch.float32)
     sel = torch.empty((n, top), dtype=torch.int32, device=h.device)
     weight = torch.empty((n, top), dtype=torch.float32, device=h.device)
-    _check(library().ia_route(_p(sel), _p(weight), _p(logits), n, E, top, ctypes.c_float(scale),
-                              SCORE_FUNCTIONS[score], int(renormalize), _stream()))
+    _check(library().ia_route(_p(sel), _p(weight), _p(h), _p(router), n, W, E, top, ctypes.c_float(scale),
+                              SCORE_FUNCTIONS[score], int(renormalize), _dt(h), _stream()))
     return sel, weight
 
 
+def tile_weights(w: torch.Tensor) -> torch.Tensor:
+    """[..., features, k] -> [..., ceil(features / 64), ceil(k / 64), 64, 64], zero-padded: the layout that the routed
+    experts' matrix-core products read (a tile of 64 features x 64 k values is 8 KB in one piece)."""
+    *lead, f, k = w.shape
+    fb, kc = -(-f // 64), -(-k // 64)
+    padded = torch.zeros((*lead, fb * 64, kc * 64), dtype=w.dtype, device=w.device)
+    padded[..., :f, :k] = w
+    return padded.view(*lead, fb, 64, kc, 64).transpose(-3, -2).contiguous()
+
+
+def experts_tiled_fits(dtype: torch.dtype, width: int, ff: int) -> bool:
+    """Whether the routed experts run on the matrix cores over tiled weights."""
+    return dtype == torch.bfloat16 and width % 8 == 0 and ff % 8 == 0
+
+
 def experts_forward(h: torch.Tensor, sel: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor,
-                    limit: float, alpha: float) -> torch.Tensor:
-    """The chosen experts of every row: w_gate_up [E, 2 ff, width] (gate rows, then up rows), w_down [E, width, ff];
+                    limit: float, alpha: float, ff: Optional[int] = None) -> torch.Tensor:
+    """The chosen experts of every row: w_gate_up [E, 2 ff, width] (gate rows, then up rows), w_down [E, width, ff],
+    or both as tiles (`tile_weights` of [E, 2, ff, width] and of [E, width, ff]; then `ff` is given);
     act = g' * sigmoid(alpha g') * (u' + 1) with g' = min(g, limit), u' = clamp(u, -limit, limit).  Returns one
     32-bit output row a (row, k) pair, [n, top, width]; nothing is added up here."""
     _dev(h, sel, w_gate_up, w_down); _i32(sel, "sel")
     n, W = h.shape
     top = sel.shape[1]
-    E, ff2, W2 = w_gate_up.shape
-    ff = ff2 // 2
-    if (W2 != W or ff2 != 2 * ff or tuple(w_down.shape) != (E, W, ff) or w_gate_up.dtype != h.dtype
-            or w_down.dtype != h.dtype or sel.shape[0] != n or E > MAX_EXPERTS):
-        raise KernelError(f"experts: weights {tuple(w_gate_up.shape)} / {tuple(w_down.shape)} do not fit rows {tuple(h.shape)}")
+    tiled = w_gate_up.dim() == 6
+    E = w_gate_up.shape[0]
+    if tiled:
+        if (ff is None or not experts_tiled_fits(h.dtype, W, ff) or w_gate_up.dtype != h.dtype or w_down.dtype != h.dtype
+                or tuple(w_gate_up.shape) != (E, 2, -(-ff // 64), -(-W // 64), 64, 64)
+                or tuple(w_down.shape) != (E, -(-W // 64), -(-ff // 64), 64, 64)):
+            raise KernelError(f"experts: tiled weights {tuple(w_gate_up.shape)} / {tuple(w_down.shape)} do not fit rows "
+                              f"{tuple(h.shape)} {h.dtype} and {ff} features an expert")
+    else:
+        ff2, W2 = w_gate_up.shape[1:]
+        ff = ff2 // 2
+        if (W2 != W or ff2 != 2 * ff or tuple(w_down.shape) != (E, W, ff) or w_gate_up.dtype != h.dtype
+                or w_down.dtype != h.dtype):
+            raise KernelError(f"experts: weights {tuple(w_gate_up.shape)} / {tuple(w_down.shape)} do not fit rows {tuple(h.shape)}")
+    if sel.shape[0] != n or E > MAX_EXPERTS:
+        raise KernelError(f"experts: {tuple(sel.shape)} choices for {n} rows, {E} experts")
     pairs = n * top
     tiles = -(-pairs // ROW_TILE) + min(E, pairs)
+    # many rows an expert: the matrix cores' large tiles (64 rows x 128 features)
+    tile = LARGE_TILE if tiled and pairs >= LARGE_TILE_FROM * LARGE_TILE * E else ROW_TILE
     lib = library()
     plan = torch.empty((pairs + 3 * tiles + 1,), dtype=torch.int32, device=h.device)
     order, t_exp, t_first, t_rows, meta = (plan[:pairs], plan[pairs:pairs + tiles], plan[pairs + tiles:pairs + 2 * tiles],
                                            plan[pairs + 2 * tiles:pairs + 3 * tiles], plan[pairs + 3 * tiles:])
-    _check(lib.ia_route_plan(_p(order), _p(t_exp), _p(t_first), _p(t_rows), _p(meta), _p(sel), pairs, E, _stream()))
+    _check(lib.ia_route_plan(_p(order), _p(t_exp), _p(t_first), _p(t_rows), _p(meta), _p(sel), pairs, E, tile, _stream()))
     act = torch.empty((pairs, ff), dtype=h.dtype, device=h.device)
     _check(lib.ia_experts_gate_up(_p(act), _p(h), _p(w_gate_up), _p(order), _p(t_exp), _p(t_first), _p(t_rows), _p(meta),
-                                  pairs, E, top, W, ff, ctypes.c_float(limit), ctypes.c_float(alpha), _dt(h), _stream()))
+                                  pairs, E, top, W, ff, ctypes.c_float(limit), ctypes.c_float(alpha), tile, int(tiled),
+                                  _dt(h), _stream()))
     y = torch.empty((n, top, W), dtype=torch.float32, device=h.device)
     _check(lib.ia_experts_down(_p(y), _p(act), _p(w_down), _p(order), _p(t_exp), _p(t_first), _p(t_rows), _p(meta), pairs,
-                               E, W, ff, _dt(h), _stream()))
+                               E, W, ff, tile, int(tiled), _dt(h), _stream()))
     return y

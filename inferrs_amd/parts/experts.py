@@ -56,11 +56,18 @@ class RoutedExperts(FeedForward):
         # the router's logits are 32-bit sums whatever its matrix is stored in (`ops.route`)
         self.router = to_compute(tensors["router"], dtype, device)
         E = spec.experts
-        self.gate_up = torch.stack([torch.cat([to_compute(tensors[f"e{e}.gate"], dtype, device),
-                                               to_compute(tensors[f"e{e}.up"], dtype, device)], dim=0) for e in range(E)]).contiguous()
-        self.down = torch.stack([to_compute(tensors[f"e{e}.down"], dtype, device) for e in range(E)]).contiguous()
+        gate_up = torch.stack([torch.cat([to_compute(tensors[f"e{e}.gate"], dtype, device),
+                                          to_compute(tensors[f"e{e}.up"], dtype, device)], dim=0) for e in range(E)])
+        down = torch.stack([to_compute(tensors[f"e{e}.down"], dtype, device) for e in range(E)])
+        # bfloat16 experts whose sizes the matrix cores take keep their weights as tiles of 64 features x 64 inputs
+        self.tiled = ops.mix.experts_tiled_fits(dtype, spec.hidden, spec.intermediate)
+        if self.tiled:
+            gate_up = ops.mix.tile_weights(gate_up.view(E, 2, spec.intermediate, spec.hidden))
+            down = ops.mix.tile_weights(down)
+        self.gate_up, self.down = gate_up.contiguous(), down.contiguous()
 
     def forward(self, ctx, h):
         s = self.spec
         sel, weights = ops.route(h, self.router, s.top, s.scale, s.score, s.renormalize)
-        return RoutedRows(ops.experts_forward(h, sel, self.gate_up, self.down, s.limit, s.alpha), weights)
+        return RoutedRows(ops.experts_forward(h, sel, self.gate_up, self.down, s.limit, s.alpha,
+                                              ff=s.intermediate if self.tiled else None), weights)
