@@ -34,24 +34,25 @@ __device__ __forceinline__ void load8(const bf16_t* p, float (&v)[8]) {
     }
 }
 
-#define IA_ROUTE_GROUP 32      // experts whose sums a wave holds at a time
+#define IA_ROUTE_WAVES 4        // waves of a token's block
+#define IA_ROUTE_SHARE 8        // experts whose sums a wave holds at a time: a block takes 32 experts a round
 
-// The logits: a lane owns the features 8 lane + 512 i of the row and adds its products up in that order (32-bit
-// multiply-adds), then the lanes' sums meet in a butterfly: an order that depends on the width alone.  VEC: the width
-// is a multiple of 8 (16-byte loads); else element by element.
+// The logits: a block of four waves a token; in every round of 32 experts a wave takes eight.  A lane owns the features
+// 8 lane + 512 i of the row and adds its products up in that order (32-bit multiply-adds), then the lanes' sums meet in a
+// butterfly: an order that depends on the width alone.  The logits meet in shared memory and the first wave picks.
+// VEC: the width is a multiple of 8 (16-byte loads); else element by element.
 template <typename T, bool VEC>
-__global__ __launch_bounds__(64) void route_kernel(int* __restrict__ sel, float* __restrict__ weight,
-                                                   const T* __restrict__ h, const T* __restrict__ wr, int n, int W, int E,
-                                                   int top, float scale, int score_fn, int renorm) {
-    const int t = blockIdx.x, lane = threadIdx.x;
+__global__ __launch_bounds__(64 * IA_ROUTE_WAVES) void route_kernel(int* __restrict__ sel, float* __restrict__ weight,
+                                                                    const T* __restrict__ h, const T* __restrict__ wr, int n,
+                                                                    int W, int E, int top, float scale, int score_fn,
+                                                                    int renorm) {
+    __shared__ float logits[IA_MAX_EXPERTS];
+    const int t = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const T* row = h + (long long)t * W;
-    float z[IA_MAX_EXPERTS / IA_WAVE];             // expert e lives in lane e % 64, register e / 64
+    for (int e0 = wave * IA_ROUTE_SHARE; e0 < E; e0 += IA_ROUTE_WAVES * IA_ROUTE_SHARE) {
+        float acc[IA_ROUTE_SHARE];
 #pragma unroll
-    for (int q = 0; q < IA_MAX_EXPERTS / IA_WAVE; ++q) z[q] = -INFINITY;
-    for (int e0 = 0; e0 < E; e0 += IA_ROUTE_GROUP) {
-        float acc[IA_ROUTE_GROUP];
-#pragma unroll
-        for (int j = 0; j < IA_ROUTE_GROUP; ++j) acc[j] = 0.f;
+        for (int j = 0; j < IA_ROUTE_SHARE; ++j) acc[j] = 0.f;
         for (int c0 = lane * 8; c0 < W; c0 += IA_WAVE * 8) {
             float x[8];
             if (VEC) {
@@ -61,7 +62,7 @@ __global__ __launch_bounds__(64) void route_kernel(int* __restrict__ sel, float*
                 for (int i = 0; i < 8; ++i) x[i] = c0 + i < W ? ld(row + c0 + i) : 0.f;
             }
 #pragma unroll
-            for (int j = 0; j < IA_ROUTE_GROUP; ++j) {
+            for (int j = 0; j < IA_ROUTE_SHARE; ++j) {
                 // (an expert beyond the last reads the last one's row: no branch stands between the loads)
                 const T* w = wr + (long long)(e0 + j < E ? e0 + j : E - 1) * W + c0;
                 float wv[8];
@@ -76,13 +77,18 @@ __global__ __launch_bounds__(64) void route_kernel(int* __restrict__ sel, float*
             }
         }
 #pragma unroll
-        for (int j = 0; j < IA_ROUTE_GROUP; ++j) {
+        for (int j = 0; j < IA_ROUTE_SHARE; ++j) {
             const float total = wave_sum(acc[j]);
-            const int e = e0 + j;
-#pragma unroll
-            for (int q = 0; q < IA_MAX_EXPERTS / IA_WAVE; ++q)
-                if (e < E && e == q * IA_WAVE + lane) z[q] = total;
+            if (lane == 0 && e0 + j < E) logits[e0 + j] = total;
         }
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    float z[IA_MAX_EXPERTS / IA_WAVE];             // expert e lives in lane e % 64, register e / 64
+#pragma unroll
+    for (int q = 0; q < IA_MAX_EXPERTS / IA_WAVE; ++q) {
+        const int e = q * IA_WAVE + lane;
+        z[q] = e < E ? logits[e] : -INFINITY;
     }
     float zmax = -INFINITY, denom = 1.f;
     if (score_fn == IA_SCORE_SOFTMAX) {
@@ -292,7 +298,7 @@ extern "C" int ia_route(int* sel, float* weight, const void* h, const void* rout
     IA_CHECK(score_fn == IA_SCORE_SIGMOID || score_fn == IA_SCORE_SOFTMAX, "route: unknown score function %d", score_fn);
     if (n == 0) return 0;
     const bool vec = W % 8 == 0 && tile_mfma_aligned(h) && tile_mfma_aligned(router);
-#define IA_ROUTE(T, V) route_kernel<T, V><<<n, 64, 0, stream>>>(sel, weight, (const T*)h, (const T*)router, n, W, E, top, scale, score_fn, renorm)
+#define IA_ROUTE(T, V) route_kernel<T, V><<<n, 64 * IA_ROUTE_WAVES, 0, stream>>>(sel, weight, (const T*)h, (const T*)router, n, W, E, top, scale, score_fn, renorm)
     if (dtype == IA_F32) { if (vec) IA_ROUTE(float, true); else IA_ROUTE(float, false); }
     else { if (vec) IA_ROUTE(bf16_t, true); else IA_ROUTE(bf16_t, false); }
 #undef IA_ROUTE

@@ -15,25 +15,19 @@
 #define IA_MAX_STREAMS 8
 
 template <typename TY, typename TH>
-__global__ __launch_bounds__(256) void streams_step_kernel(
+__global__ __launch_bounds__(512) void streams_step_kernel(
     float* __restrict__ streams, const TY* __restrict__ y, const float* __restrict__ yw, int K,
     const float* __restrict__ scale, const float* __restrict__ mix, const float* __restrict__ outc,
     const float* __restrict__ inc, const float* __restrict__ w, float eps, TH* __restrict__ h,
     const int* __restrict__ rows, int S, int W) {
     extern __shared__ float u_sh[];              // [W]: the row that the norm reads
     __shared__ float scratch[16];
-    __shared__ float coef[IA_MAX_STREAMS * IA_MAX_STREAMS + 2 * IA_MAX_STREAMS];
     const int r = blockIdx.x;
     const int row = rows != nullptr ? rows[r] : r;
-    float* cm = coef;                            // mix [S][S]
-    float* co = coef + IA_MAX_STREAMS * IA_MAX_STREAMS;
-    float* ci = co + IA_MAX_STREAMS;
-    if (threadIdx.x < S * S) cm[threadIdx.x] = mix != nullptr ? mix[threadIdx.x] : 0.f;
-    if (threadIdx.x < S) {
-        co[threadIdx.x] = outc != nullptr ? outc[threadIdx.x] : 0.f;
-        ci[threadIdx.x] = inc != nullptr ? inc[threadIdx.x] : 1.f;
-    }
-    __syncthreads();
+    // (the coefficients are the same for every lane: read where they are used, they come through the scalar cache
+    // beside the row's own loads instead of a round trip ahead of them)
+    const float* cm = mix;                       // [S][S]
+    const float* co = outc;
     float* xr = streams + (long long)row * S * W;
     float sq = 0.f;
 #pragma unroll 4
@@ -69,7 +63,7 @@ __global__ __launch_bounds__(256) void streams_step_kernel(
             float u = 0.f;
 #pragma unroll
             for (int s = 0; s < IA_MAX_STREAMS; ++s)
-                if (s < S) u = fmaf(ci[s], x[s], u);
+                if (s < S) u = fmaf(inc != nullptr ? inc[s] : 1.f, x[s], u);
             u_sh[c] = u;
             sq = fmaf(u, u, sq);
         }
@@ -97,8 +91,9 @@ extern "C" int ia_streams_step(float* streams, const void* y, const float* yw, i
     IA_CHECK((size_t)W * sizeof(float) <= 60 * 1024, "streams_step: width %d does not fit shared memory", W);
     if (n == 0 || (y == nullptr && h == nullptr)) return 0;
     const size_t shm = h != nullptr ? (size_t)W * sizeof(float) : 0;
+    const int threads = W >= 2048 ? 512 : 256;
 #define IA_LAUNCH(TY, TH)                                                                                          \
-    streams_step_kernel<TY, TH><<<n, 256, shm, stream>>>(streams, (const TY*)y, yw, K, scale, mix, outc, inc, w, eps, \
+    streams_step_kernel<TY, TH><<<n, threads, shm, stream>>>(streams, (const TY*)y, yw, K, scale, mix, outc, inc, w, eps, \
                                                          (TH*)h, rows, S, W)
     if (y_dtype == IA_F32 && h_dtype == IA_F32) IA_LAUNCH(float, float);
     else if (y_dtype == IA_F32) IA_LAUNCH(float, bf16_t);

@@ -80,7 +80,10 @@ class Rotary(Position):
             if law not in SCALING_LAWS:
                 raise SpecError(f"rotary scaling {law!r} has no entry (known: {sorted(SCALING_LAWS)})")
             extra = dict(theta=float(spec.theta), rot_dim=spec.rot_dim) if law in SCALING_NEEDS_GEOMETRY else {}
-            scaled = SCALING_LAWS[law](inv_freq, *numbers, **extra)
+            try:
+                scaled = SCALING_LAWS[law](inv_freq, *numbers, **extra)
+            except TypeError:
+                raise SpecError(f"rotary scaling {law!r} does not take the {len(numbers)} numbers {numbers}") from None
             if isinstance(scaled, tuple):
                 inv_freq, self.magnitude = scaled[0], float(scaled[1])
             else:

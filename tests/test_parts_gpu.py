@@ -1048,6 +1048,9 @@ def test_position_part_with_a_scaling_law():
     cos_b, sin_b = b.table((pos * 4).to(DEV))
     assert float((cos_a - cos_b).abs().max()) < 1e-6 and float((sin_a - sin_b).abs().max()) < 1e-6
     assert torch.equal(b.inv_freq.cpu(), a.inv_freq.cpu() / 4)
-    other = PositionSpec(kind="rope", head_dim=32, rot_dim=32, theta=1e4, scaling=("yarn", 4.0))
-    with pytest.raises(SpecError, match="yarn.*linear"):
+    other = PositionSpec(kind="rope", head_dim=32, rot_dim=32, theta=1e4, scaling=("ntk", 4.0))
+    with pytest.raises(SpecError, match="ntk.*linear"):
         part_class("position", other)(other, {}, torch.float32, DEV)
+    short = PositionSpec(kind="rope", head_dim=32, rot_dim=32, theta=1e4, scaling=("yarn", 4.0))     # (the law takes four numbers)
+    with pytest.raises(SpecError, match="yarn"):
+        part_class("position", short)(short, {}, torch.float32, DEV)
