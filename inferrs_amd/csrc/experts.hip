@@ -53,6 +53,8 @@ __global__ __launch_bounds__(64 * IA_ROUTE_WAVES) void route_kernel(int* __restr
         float acc[IA_ROUTE_SHARE];
 #pragma unroll
         for (int j = 0; j < IA_ROUTE_SHARE; ++j) acc[j] = 0.f;
+        // (four rounds of loads under way at once: a round is a trip to the memory)
+#pragma unroll 4
         for (int c0 = lane * 8; c0 < W; c0 += IA_WAVE * 8) {
             float x[8];
             if (VEC) {

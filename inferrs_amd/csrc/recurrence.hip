@@ -1,5 +1,6 @@
 // A gated linear recurrence a channel (the real-gated linear recurrent unit) behind a short causal convolution:
-//     u_t = bias + sum_j taps[j] * in_(t - (k - 1 - j))                       (zeros before a sequence's start)
+//     u_t = bias + sum_j taps[j] * in_(t - (k - 1 - j))                       (zeros before a sequence's start;
+//                                                                              taps are handed over as [k][width])
 //     r_t = sigmoid(zr_t + br),  i_t = sigmoid(zi_t + bi)                    (zr, zi: block-diagonal products of u)
 //     a_t = exp(-c * r_t * softplus(lam)),   S_t = a_t S_(t-1) + sqrt(1 - a_t^2) * i_t * u_t
 //     out_t = S_t * gelu_tanh(branch_t)
@@ -28,10 +29,21 @@ __global__ void conv_step_kernel(float* __restrict__ u, bf16_t* __restrict__ u_l
         float v;
         if (src >= first) v = ld(x + (long long)src * x_ld + x_off + c);
         else v = tail[(long long)((k - 1) + (src - first)) * width];
-        acc = fmaf(ld(taps + (long long)c * k + j), v, acc);
+        acc = fmaf(ld(taps + (long long)j * width + c), v, acc);
     }
     u[i] = acc;
     if (u_lo != nullptr) st(u_lo + i, acc);
+}
+
+// eight neighbouring bfloat16 values (16-byte aligned) as 32-bit floats
+typedef uint32_t rec_u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void unpack8(const bf16_t* p, float (&v)[8]) {
+    const rec_u32x4 q = *reinterpret_cast<const rec_u32x4*>(p);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        v[2 * e] = __uint_as_float(q[e] << 16);
+        v[2 * e + 1] = __uint_as_float(q[e] & 0xffff0000u);
+    }
 }
 
 // The same for bfloat16 rows, eight neighbouring channels a thread (16-byte loads of the rows, two 16-byte stores of u
@@ -49,26 +61,24 @@ __global__ void conv_step8_kernel(float* __restrict__ u, bf16_t* __restrict__ u_
     const int first = cu_tokens[seq];
     const float* tail = state + ((long long)state_slots[seq] * k + 1) * width + c;
     float acc[8];
+    if (bias != nullptr) unpack8(bias + c, acc);
+    else {
 #pragma unroll
-    for (int e = 0; e < 8; ++e) acc[e] = bias != nullptr ? ld(bias + c + e) : 0.f;
+        for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    }
     for (int j = 0; j < k; ++j) {
         const int src = t - (k - 1 - j);
-        float v[8];
+        float v[8], tp[8];
+        unpack8(taps + (long long)j * width + c, tp);
         if (src >= first) {
-            const uint4 p = *reinterpret_cast<const uint4*>(x + (long long)src * x_ld + x_off + c);
-            const uint32_t w[4] = {p.x, p.y, p.z, p.w};
-#pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                v[2 * e] = __uint_as_float(w[e] << 16);
-                v[2 * e + 1] = __uint_as_float(w[e] & 0xffff0000u);
-            }
+            unpack8(x + (long long)src * x_ld + x_off + c, v);
         } else {
             const float* from = tail + (long long)((k - 1) + (src - first)) * width;
 #pragma unroll
             for (int e = 0; e < 8; ++e) v[e] = from[e];
         }
 #pragma unroll
-        for (int e = 0; e < 8; ++e) acc[e] = fmaf(ld(taps + (long long)(c + e) * k + j), v[e], acc[e]);
+        for (int e = 0; e < 8; ++e) acc[e] = fmaf(tp[e], v[e], acc[e]);
     }
     float* out = u + (long long)t * width + c;
     *reinterpret_cast<float4*>(out) = make_float4(acc[0], acc[1], acc[2], acc[3]);

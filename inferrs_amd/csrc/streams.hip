@@ -77,6 +77,78 @@ __global__ __launch_bounds__(512) void streams_step_kernel(
     }
 }
 
+// The same for rows of up to 4,096 features: a thread owns up to four columns and asks for everything it reads (the
+// streams, the output, scales, the norm's weight) before it stores anything, so that one trip to the memory serves the
+// whole step; the kernel above updates the streams in place column by column, and a column's loads cannot pass the
+// stores of the column before.  The arithmetic and its order are those of the kernel above.
+#define IA_STREAMS_COLS 4
+
+template <typename TY, typename TH>
+__global__ __launch_bounds__(1024) void streams_step_rows_kernel(
+    float* __restrict__ streams, const TY* __restrict__ y, const float* __restrict__ yw, int K,
+    const float* __restrict__ scale, const float* __restrict__ mix, const float* __restrict__ outc,
+    const float* __restrict__ inc, const float* __restrict__ w, float eps, TH* __restrict__ h,
+    const int* __restrict__ rows, int S, int W) {
+    __shared__ float scratch[16];
+    const int r = blockIdx.x, tid = threadIdx.x, nt = blockDim.x;
+    const int row = rows != nullptr ? rows[r] : r;
+    float* xr = streams + (long long)row * S * W;
+    float x[IA_STREAMS_COLS][IA_MAX_STREAMS], yv[IA_STREAMS_COLS], wn[IA_STREAMS_COLS];
+#pragma unroll
+    for (int i = 0; i < IA_STREAMS_COLS; ++i) {
+        const int c = tid + i * nt;
+        const bool in = c < W;
+#pragma unroll
+        for (int s = 0; s < IA_MAX_STREAMS; ++s) x[i][s] = (in && s < S) ? xr[(long long)s * W + c] : 0.f;
+        yv[i] = 0.f;
+        if (y != nullptr && in) {
+            if (yw != nullptr) {
+                for (int k = 0; k < K; ++k)
+                    yv[i] = fmaf(yw[(long long)row * K + k], ld(y + ((long long)row * K + k) * W + c), yv[i]);
+            } else {
+                yv[i] = ld(y + (long long)row * W + c);
+            }
+            if (scale != nullptr) yv[i] *= scale[c];
+        }
+        wn[i] = (h != nullptr && w != nullptr && in) ? w[c] : 1.f;
+    }
+    float u[IA_STREAMS_COLS];
+    float sq = 0.f;
+#pragma unroll
+    for (int i = 0; i < IA_STREAMS_COLS; ++i) {
+        const int c = tid + i * nt;
+        const bool in = c < W;
+        if (y != nullptr) {
+            float nx[IA_MAX_STREAMS];
+#pragma unroll
+            for (int t = 0; t < IA_MAX_STREAMS; ++t) {
+                float v = 0.f;
+                if (t < S) {
+                    for (int s = 0; s < S; ++s) v = fmaf(mix[s * S + t], x[i][s], v);
+                    v = fmaf(outc[t], yv[i], v);
+                    if (in) xr[(long long)t * W + c] = v;
+                }
+                nx[t] = v;
+            }
+#pragma unroll
+            for (int t = 0; t < IA_MAX_STREAMS; ++t) x[i][t] = nx[t];
+        }
+        u[i] = 0.f;
+#pragma unroll
+        for (int s = 0; s < IA_MAX_STREAMS; ++s)
+            if (s < S) u[i] = fmaf(inc != nullptr ? inc[s] : 1.f, x[i][s], u[i]);
+        if (in) sq = fmaf(u[i], u[i], sq);
+    }
+    if (h == nullptr) return;
+    const float total = block_sum(sq, scratch);
+    const float rs = 1.0f / sqrtf(total / (float)W + eps);
+#pragma unroll
+    for (int i = 0; i < IA_STREAMS_COLS; ++i) {
+        const int c = tid + i * nt;
+        if (c < W) st(h + (long long)r * W + c, u[i] * rs * wn[i]);
+    }
+}
+
 // y_dtype / h_dtype: 0 float32, 1 bfloat16.  y null: nothing is written to the streams; h null: nothing is read for
 // a next sub-layer.  rows null: every row 0..n-1; else the n rows named (only for a call without y).
 extern "C" int ia_streams_step(float* streams, const void* y, const float* yw, int K, const float* scale,
@@ -92,13 +164,19 @@ extern "C" int ia_streams_step(float* streams, const void* y, const float* yw, i
     if (n == 0 || (y == nullptr && h == nullptr)) return 0;
     const size_t shm = h != nullptr ? (size_t)W * sizeof(float) : 0;
     const int threads = W >= 2048 ? 512 : 256;
-#define IA_LAUNCH(TY, TH)                                                                                          \
-    streams_step_kernel<TY, TH><<<n, threads, shm, stream>>>(streams, (const TY*)y, yw, K, scale, mix, outc, inc, w, eps, \
-                                                         (TH*)h, rows, S, W)
-    if (y_dtype == IA_F32 && h_dtype == IA_F32) IA_LAUNCH(float, float);
-    else if (y_dtype == IA_F32) IA_LAUNCH(float, bf16_t);
-    else if (h_dtype == IA_F32) IA_LAUNCH(bf16_t, float);
-    else IA_LAUNCH(bf16_t, bf16_t);
+    const bool few = W <= 1024 * IA_STREAMS_COLS;
+    const int row_threads = ((W + IA_STREAMS_COLS - 1) / IA_STREAMS_COLS + 63) / 64 * 64;
+#define IA_LAUNCH(TY, TH)                                                                                              \
+    if (few)                                                                                                           \
+        streams_step_rows_kernel<TY, TH><<<n, row_threads, 0, stream>>>(streams, (const TY*)y, yw, K, scale, mix, outc,   \
+                                                                        inc, w, eps, (TH*)h, rows, S, W);                \
+    else                                                                                                               \
+        streams_step_kernel<TY, TH><<<n, threads, shm, stream>>>(streams, (const TY*)y, yw, K, scale, mix, outc, inc, w,  \
+                                                                 eps, (TH*)h, rows, S, W)
+    if (y_dtype == IA_F32 && h_dtype == IA_F32) { IA_LAUNCH(float, float); }
+    else if (y_dtype == IA_F32) { IA_LAUNCH(float, bf16_t); }
+    else if (h_dtype == IA_F32) { IA_LAUNCH(bf16_t, float); }
+    else { IA_LAUNCH(bf16_t, bf16_t); }
 #undef IA_LAUNCH
     IA_LAUNCH_CHECK("streams_step");
     return 0;

@@ -151,12 +151,13 @@ def conv_step(x: torch.Tensor, x_off: int, width: int, taps: torch.Tensor, bias:
               state: torch.Tensor, token_seq: torch.Tensor, cu_tokens: torch.Tensor,
               state_slots: torch.Tensor, rounded: bool = False):
     """The causal convolution a channel over the step's tokens: x[:, x_off : x_off + width] -> 32-bit u
-    [n, width]; inputs before a request's portion come from rows 1.. of its state row ([slots, k, width]).
+    [n, width]; `taps` [k, width] (tap by tap, the last meets the current token); inputs before a request's portion
+    come from rows 1.. of its state row ([slots, k, width]).
     `rounded`: returns (u, its bfloat16 copy)."""
     _dev(x, taps, bias, state, token_seq, cu_tokens, state_slots); _f32(state, "state")
     _i32(token_seq, "token_seq"); _i32(cu_tokens, "cu_tokens"); _i32(state_slots, "state_slots")
-    n, k = x.shape[0], taps.shape[1]
-    if (tuple(taps.shape) != (width, k) or taps.dtype != x.dtype or state.dim() != 3
+    n, k = x.shape[0], taps.shape[0]
+    if (tuple(taps.shape) != (k, width) or taps.dtype != x.dtype or state.dim() != 3
             or tuple(state.shape[1:]) != (k, width) or (bias is not None and (bias.numel() != width or bias.dtype != x.dtype))):
         raise KernelError(f"conv_step: taps {tuple(taps.shape)} / state {tuple(state.shape)} do not fit width {width}")
     u = torch.empty((n, width), dtype=torch.float32, device=x.device)

@@ -50,7 +50,7 @@ class GatedRecurrence(Mixer):
             raise SpecError(f"rglru: width {spec.width} in {spec.blocks} blocks, {spec.conv} taps")
         self.spec = spec
         self.proj = Linear([tensors["y"], tensors["x"]], dtype, device, [tensors["y.b"], tensors["x.b"]])
-        self.taps = to_compute(tensors["conv"], dtype, device)
+        self.taps = to_compute(tensors["conv"], dtype, device).t().contiguous()          # [taps, width]: the kernels read tap by tap
         self.conv_bias = to_compute(tensors["conv.b"], dtype, device)
         # a block's two gate matrices one above the other: [blocks, 2 bw, bw]
         self.gates = torch.cat([to_compute(tensors["ra"], dtype, device), to_compute(tensors["ri"], dtype, device)], dim=1).contiguous()

@@ -58,7 +58,13 @@ CFG_D = {"architecture": "Buketar", "vocab": 150, "width": 64, "norm": {"eps": 1
          "layers": [layer(attention(8, 16, 32, 24, 96, 0.15, base=100.0, scaling={"factor": 16.0, "original": 32, "fast": 4.0, "slow": 2.0}),
                           moe(40, 6, 3, 2.0, 1.0)),
                     layer(attention(2, 40, 16, 8, 16, 0.1, base=1e6, turned=16), moe(40, 6, 3, 2.0, 1.0))]}
-CONFIGS = {"A": CFG_A, "B": CFG_B, "C": CFG_C, "D": CFG_D}
+# E: sizes that fit no vector width: a model width of 50, experts of 30, a recurrence of 42 channels in blocks of 14, a
+# cached row of 28, five heads, three streams, seven experts of which a token runs five.
+CFG_E = {"architecture": "Buketar", "vocab": 101, "width": 50, "norm": {"eps": 1e-5}, "streams": 3, "logit_softcap": 20.0,
+         "loop": {"start": 1, "stop": 2, "times": 2},
+         "layers": [layer(attention(5, 12, 6, 10, 22, 0.25, base=777.0, turned=2), moe(30, 7, 5, 1.2, 1.5)),
+                    layer(recurrence(42, 3, 3), moe(30, 7, 5, 1.2, 1.5))]}
+CONFIGS = {"A": CFG_A, "B": CFG_B, "C": CFG_C, "D": CFG_D, "E": CFG_E}
 
 
 def tensor_shapes(cfg: dict) -> Dict[str, tuple]:

@@ -32,7 +32,7 @@ pytestmark = pytest.mark.gpu
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 LENGTHS = [1, 2, 3, 17, 64, 65, 130, 300, 700]
 TOL_F32 = 2e-5
-CASES = [("A", 1.0), ("B", 1.0), ("C", 1.0), ("D", 1.0), ("A", 4.0), ("B", 6.0), ("D", 4.0)]
+CASES = [("A", 1.0), ("B", 1.0), ("C", 1.0), ("D", 1.0), ("E", 1.0), ("A", 4.0), ("B", 6.0), ("D", 4.0)]
 
 
 def dev(t, dtype=None):
@@ -166,8 +166,8 @@ def test_recurrence_carried_over_portions(width, blocks, taps, chunked):
         cu = dev(torch.tensor([0] + list(np.cumsum(counts)), dtype=torch.int32))
         seq = dev(torch.tensor([i for i, c in enumerate(counts) for _ in range(c)], dtype=torch.int32))
         slots = dev(torch.tensor(live, dtype=torch.int32))
-        u = ops.conv_step(rows, width, width, dev(w["conv"]), dev(w["conv.b"]), state, seq, cu, slots)
-        assert ops.conv_step(rows, width, width, dev(w["conv"]), dev(w["conv.b"]), state, seq, cu, slots, rounded=True)[1].dtype == torch.bfloat16
+        u = ops.conv_step(rows, width, width, dev(w["conv"].t()), dev(w["conv.b"]), state, seq, cu, slots)
+        assert ops.conv_step(rows, width, width, dev(w["conv"].t()), dev(w["conv.b"]), state, seq, cu, slots, rounded=True)[1].dtype == torch.bfloat16
         z = ops.head_product(u, gates, out_dtype=torch.float32)
         out = ops.rglru_scan(u, z, rows, branch_off=0, x_off=width, bias_r=dev(w["ra.b"].reshape(-1)), bias_i=dev(w["ri.b"].reshape(-1)),
                              lam=dev(w["lam"]), state=state, cu_tokens=cu, state_slots=slots, block_width=bw, decay=8.0, chunked=chunked)
