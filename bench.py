@@ -18,6 +18,13 @@ choice): `mixed16` is 16 requests with prompts of 128 to 4,096 random tokens in 
 `--decode-tokens` tokens.  Its JSON line gives tokens a second over the whole run, the prompts' and the
 decoded tokens' rates apart, and the time to a request's first token.
 
+    python bench.py --design buketar [--design-shapes 1k,2k,4k]
+
+measures the Buketar design (latent attention, gated recurrences, routed experts, residual streams) at a few layer
+sizes beside the dense decoder at equal width, layers and feed-forward products a token: prompts of `--prefill-tokens`
+tokens, decode steps at `--batch` and at batch 1 through the serving loop, and every kernel's time in one prompt and one
+decode step of both.  One JSON line; the default record above is not touched by it.
+
 The reference measures the same quantities with `inferrs bench` (`inferrs/src/bench.rs:40-224`,
 `Engine::bench_generate`, `inferrs/src/engine.rs:2557-2641`): synthetic prompt, stop tokens
 ignored, device-synchronised wall time.

@@ -183,9 +183,9 @@ extern "C" int ia_head_product(void* out, const void* x, const void* w, const vo
                                                               g_ld, g_off)
     const bool cores = x_dtype == IA_BF16 && w_dtype == IA_BF16 && k_in % 8 == 0 && x_ld % 8 == 0 && x_off % 8 == 0 &&
                        x_head % 8 == 0 && tile_mfma_aligned(x) && tile_mfma_aligned(w);
+    // many rows and wide heads: tiles of 64 rows x 128 features (every operand read serves more products)
     const bool large = n >= 64 && n_out >= 128;
     const dim3 big((n_out + 127) / 128, (n + 63) / 64, H);
-    (void)big;
 #define IA_CORES(TO, RT, FT, KC, G)                                                                                            \
     head_product_mfma_kernel<TO, RT, FT, KC><<<G, 256, 0, stream>>>((TO*)out, (const bf16_t*)x, (const bf16_t*)w,                 \
                                                                     (const bf16_t*)gate, n, n_out, k_in, x_ld, x_off, x_head,    \
