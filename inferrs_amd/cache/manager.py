@@ -18,7 +18,7 @@ from dataclasses import dataclass
 from typing import Dict, Hashable, Iterator, List, Optional, Sequence, Tuple
 
 from .. import native
-from ..parts.base import FixedState, PagedKV
+from ..parts.base import FixedState, PagedAndState, PagedKV
 
 RELEASED = native.RELEASED
 
@@ -220,7 +220,10 @@ def group_layers(needs: Dict[int, object]) -> Tuple[List[Tuple[PagedKV, List[int
         need = needs[layer]
         if need is None:
             continue
-        if isinstance(need, PagedKV):
+        if isinstance(need, PagedAndState):
+            groups.setdefault(need.paged, []).append(layer)
+            states.append(StateInfo(layer, need.state))
+        elif isinstance(need, PagedKV):
             groups.setdefault(need, []).append(layer)
         elif isinstance(need, FixedState):
             states.append(StateInfo(layer, need))
@@ -231,7 +234,7 @@ def group_layers(needs: Dict[int, object]) -> Tuple[List[Tuple[PagedKV, List[int
 
 class CacheManager:
     def __init__(self, needs: Dict[int, object], page_size: int, num_pages, max_seqs: int):
-        """`needs`: cache-owning layer -> PagedKV | FixedState | None.
+        """`needs`: cache-owning layer -> PagedKV | FixedState | PagedAndState | None.
         `num_pages`: an int for every group, or a list with one entry per group."""
         if page_size < 1:
             raise CacheError(f"page_size must be >= 1, got {page_size}")

@@ -12,7 +12,8 @@ page_size, value_dim]` (`value_layout="rows"`), or for no value array at all (`v
 attention kernels read pages through the block table.)  Pages are not cleared on reuse:
 attention never reads beyond a request's length.
 
-State layers: one array `[max_seqs, *shape]`; a request's row is cleared when its slot is handed out.
+State layers: one array `[max_seqs, *shape]`; a request's row is cleared when its slot is handed out.  A layer
+whose mixer keeps both (`PagedAndState`) has `k`, `v` and `state` in one `LayerCache`.
 """
 from __future__ import annotations
 
@@ -67,7 +68,10 @@ class CacheStorage:
         for st in manager.states:
             arr = torch.zeros((manager.max_seqs, *st.need.shape), dtype=st.need.dtype, device=device)
             self.arrays.append(arr)
-            self.layers[st.layer] = LayerCache(st.layer, state=arr)
+            if st.layer in self.layers:              # a mixer that keeps pages and a state
+                self.layers[st.layer].state = arr
+            else:
+                self.layers[st.layer] = LayerCache(st.layer, state=arr)
 
     def clear_state_slot(self, slot: int) -> None:
         for st in self.manager.states:

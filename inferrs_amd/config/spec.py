@@ -66,6 +66,9 @@ class AttentionSpec:
     scale: Optional[float] = None          # None = 1/sqrt(head_dim)
     qkv_bias: bool = False                 # q_proj.bias, k_proj.bias, v_proj.bias are added to the projections
     o_bias: bool = False                   # o_proj.bias is added to the output projection
+    sink: bool = False                     # the softmax's denominator holds one more term, exp(0): a key of score 0 without a value
+    values_from_keys: bool = False         # no value projection: a value is its key as projected, before norm and rotation
+    names: Optional[Tuple[Tuple[str, str], ...]] = None    # (the part's tensor name, the name in the file) where they differ
     kind: str = "attention"
 
     @property
@@ -82,6 +85,86 @@ class GatedMlpSpec:
     activation: str = "silu"
     bias: bool = False
     kind: str = "gated_mlp"
+
+
+@dataclass(frozen=True)
+class DenseMlpSpec:
+    """down( act(up(x)) ), no gate and no biases.  `activation`: "gelu" (the exact one), "gelu_tanh" or "silu"."""
+    hidden: int
+    intermediate: int
+    activation: str = "gelu"
+    kind: str = "dense_mlp"
+
+
+@dataclass(frozen=True)
+class RetentionSpec:
+    """Linear attention with a fixed decay a head and neither softmax nor denominator: k is scaled by dim^-1/2,
+    S <- decay_h S + k v^T, o = S^T q; each head's o is divided by its root mean square (`norm_eps`, no weight), the
+    joined heads are multiplied by silu(W_g h) and projected.  No biases."""
+    hidden: int
+    n_heads: int
+    head_dim: int
+    v_dim: int
+    decay: Tuple[float, ...]
+    norm_eps: float
+    kind: str = "retention"
+
+
+@dataclass(frozen=True)
+class SideBySideSpec:
+    """Two mixers that read the same input; the result is left_scale * left + right_scale * right.  Their tensors
+    lie under `left_prefix` and `right_prefix` of the layer's mixer."""
+    left: Any
+    right: Any
+    left_scale: float = 1.0
+    right_scale: float = 1.0
+    left_prefix: str = "left."
+    right_prefix: str = "right."
+    kind: str = "side_by_side"
+
+
+@dataclass(frozen=True)
+class MatrixMemorySpec:
+    """The matrix memory with exponential gates (the mLSTM of the xLSTM): q is scaled by dim^-1/2; a log input gate
+    i = cap tanh((W_i h + b_i) / cap) and a log forget gate f = logsigmoid(cap tanh((W_f h + b_f) / cap)) a head; under a
+    running maximum m_t = max(f + m_(t-1), i) that starts at 0, S <- exp(f + m_(t-1) - m_t) S + exp(i - m_t) k v^T and
+    n likewise with k alone; o = S^T q / (max(|n . q|, exp(-m_t)) + 1e-6); each head's o is divided by its root mean
+    square (`norm_eps`), the joined heads times a weight, times sigmoid(W_g h), projected."""
+    hidden: int
+    n_heads: int
+    head_dim: int
+    v_dim: int
+    gate_cap: float
+    norm_eps: float
+    kind: str = "mlstm"
+
+
+@dataclass(frozen=True)
+class StateSpaceSpec:
+    """A selective state space with a scalar decay a head (Mamba-2): one product gives [z | x | B | C | dt] with
+    inner = n_heads * v_dim and `groups` groups of `state` entries for B and C; x, B and C pass a causal convolution a
+    channel (`conv` taps, a bias) and SiLU; dt = softplus(dt + dt_bias); S <- exp(-exp(A_log) dt) S + dt B x^T,
+    y = S^T C + D x; y * silu(z) is RMS-normed in `norm_groups` equal parts (`norm_eps`), times a weight, projected."""
+    hidden: int
+    n_heads: int
+    v_dim: int
+    state: int
+    groups: int
+    conv: int
+    norm_groups: int
+    norm_eps: float
+    kind: str = "mamba2"
+
+
+@dataclass(frozen=True)
+class PassInputSpec:
+    """What enters the stream before each pass over a looped range of layers: row t of the tensor `name` [times,
+    hidden] before pass t, and, before every pass but the first, the embedding's output once more (`readd_embedding`)."""
+    name: str
+    times: int
+    hidden: int
+    readd_embedding: bool = True
+    kind: str = "pass_input"
 
 
 @dataclass(frozen=True)
@@ -158,7 +241,9 @@ class LayerSpec:
 
     `arrangement` names a registered block class (`parts.register_block`), which says how many
     norms it has and where they stand: "pre_norm" has two, before the mixer and before the
-    feed-forward; "streams" is pre-norm around several residual streams (`residual`: a `StreamsSpec`) and takes a
+    feed-forward; "sandwich_norm" has a norm before and a norm behind each sub-layer around a 32-bit stream (norms in the
+    order before the mixer, behind it, before the feed-forward, behind it; two norms for a layer without a feed-forward);
+    "streams" is pre-norm around several residual streams (`residual`: a `StreamsSpec`) and takes a
     layer without a feed-forward (`ffn` None, one norm).  `norms[i]` loads its weight from `norm_names[i]`."""
     mixer: Any
     ffn: Any
@@ -213,6 +298,7 @@ class ScheduleEntry:
     """
     layer: int
     cache_of: Optional[int] = None
+    pass_index: Optional[int] = None    # this stop begins pass t of a looped range: `ModelSpec.pass_input` enters before it
 
 
 @dataclass(frozen=True)
@@ -231,6 +317,7 @@ class ModelSpec:
     eos_token_ids: Tuple[int, ...] = field(default_factory=tuple)
     embedding: Any = None               # a spec whose `kind` names a registered embedding part; None: EmbeddingSpec
     head: Any = None                    # likewise for the logits head; None: HeadSpec
+    pass_input: Any = None              # a spec whose `kind` names a registered pass-input part (stops with a `pass_index`)
 
     def __post_init__(self):
         if self.embedding is None:

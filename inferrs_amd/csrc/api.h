@@ -43,12 +43,13 @@ int ia_qk_rope_kv(void* q_out, void* k_cache, void* v_cache, const void* qkv,
                   int interleaved, int page_size, float eps, int add_one, int dtype,
                   hipStream_t stream);
 
+// sink: 1 adds exp(0) to the softmax's denominator (a key of score 0 that has no value); the same in the matrix-core kernels.
 // workspace: null, or ia_attention_generic_workspace(...) floats when that is not 0 (steps of few tokens: a wave a
 // segment of keys and a merge kernel, the same bits as without); max_kv_len: an upper bound of positions + 1
 int ia_attention_generic(void* out, const void* q, const void* k_cache, const void* v_cache,
                          const int* positions, const int* token_seq, const int* block_table,
                          int n, int max_pages, int nq, int nkv, int d, int page_size, int window,
-                         float scale, int dtype, float* workspace, int max_kv_len, hipStream_t stream);
+                         float scale, int dtype, float* workspace, int max_kv_len, int sink, hipStream_t stream);
 long long ia_attention_generic_workspace(int n, int nq, int nkv, int d, int max_kv_len);
 
 int ia_gemm_tiled(void* out, const void* x, const void* w, int M, int N, int K, int in_dtype,
@@ -189,6 +190,40 @@ int ia_experts_down(float* y, const void* act, const void* w_down, const int* or
                     const int* tile_first, const int* tile_rows, const int* meta, int pairs, int E, int W,
                     int ff, int tile, int tiled, int dtype, hipStream_t stream);
 
+// A 32-bit residual stream whose sub-layers stand between two norms (sandwich.hip): x += rmsnorm(s1 y1 + s2 y2) * w_post;
+// x += e_rows + e_vec; h = rmsnorm(x) * w_pre.  Every half may be null.  With `rows` only the named rows are read and the
+// stream is not written.  y_dtype: precision of y1, y2, e_rows; h_dtype: of h.
+int ia_sandwich_step(float* x, const void* y1, float s1, const void* y2, float s2, const float* w_post,
+                     const void* e_rows, const float* e_vec, const float* w_pre, float eps_post, float eps, void* h,
+                     const int* rows, int n, int W, int y_dtype, int h_dtype, hipStream_t stream);
+// act over every element in place: 1 SiLU, 2 GELU in its tanh form, 3 the exact GELU
+int ia_activation(void* x, long long n, int act, int dtype, hipStream_t stream);
+// Mixers with a matrix state a head (linear_state.hip).  A request's state is its row of `state` [slots][row_floats];
+// every kernel takes the offset of its part of the row.
+int ia_conv_act_step(void* out, const void* x, const void* taps, const void* bias, float* state,
+                     long long row_floats, long long tail_off, const int* token_seq, const int* cu_tokens,
+                     const int* state_slots, int n, int n_seqs, int C, int k, long long x_ld, int x_off, int act,
+                     int dtype, hipStream_t stream);
+int ia_exp_gates(float* log_a, float* b, float* floor_, float* state, long long row_floats, long long m_off,
+                 const void* proj, long long p_ld, int i_off, int f_off, const float* bias_i,
+                 const float* bias_f, float cap, const int* cu_tokens, const int* state_slots, int H,
+                 int n_seqs, int dtype, hipStream_t stream);
+int ia_step_gates(float* log_a, float* b, const void* proj, long long p_ld, int dt_off, const float* dt_bias,
+                  const float* a_log, int n, int H, int dtype, hipStream_t stream);
+// S <- a S + b k v^T, o = S^T q (+ skip v); `den` not null: one more column of S whose value is always 1.
+// log_a: [n][H] logarithms of the decays (a_per_token 1) or the decays themselves, [H] (a_per_token 0).
+int ia_linear_scan(float* out, float* den, float* state, long long row_floats, long long s_off,
+                   const void* q, long long q_ld, int q_off, int q_heads,
+                   const void* k, long long k_ld, int k_off, int k_heads,
+                   const void* v, long long v_ld, int v_off,
+                   const float* log_a, int a_per_token, const float* b, const float* skip,
+                   const int* cu_tokens, const int* state_slots, int n_seqs, int H, int dim, int vdim,
+                   float q_scale, float k_scale, int dtype, hipStream_t stream);
+// [o / (max(|den|, floor) + 1e-6)] [* act(gate)] -> RMS norm in groups of `group` features [* w] [* act(gate)]; act: 1 SiLU, 4 sigmoid
+int ia_group_norm_gate(void* out, const float* o, const float* den, const float* floor_, int head,
+                       const void* gate, long long g_ld, int g_off, int act, int gate_first, const float* w,
+                       float eps, int n, int inner, int group, int dtype, hipStream_t stream);
+
 // Built per head size (-DIA_HEAD_DIM) into a library of its own.
 int ia_attention_mfma_head_dim(void);
 long long ia_attention_mfma_workspace(int n, int nq, int splits);
@@ -197,7 +232,7 @@ int ia_attention_mfma(void* out, float* workspace, const void* q, const void* k_
                       const int* positions, int n, int seq_begin, int n_seqs, int token_begin,
                       int n_tokens, int max_q_len, int max_kv_len, int max_pages,
                       int nq, int nkv, int d, int page_size, int window, float scale,
-                      int splits, int chunk, hipStream_t stream);
+                      int splits, int chunk, int sink, hipStream_t stream);
 // Decode steps (one token a request, head sizes in steps of 64): per-head norm, rotation, cache write, attention
 // and the merge of the key splits in one kernel.  `workspace` holds ia_attention_decode_workspace() floats;
 // `counters` holds at least ia_attention_decode_counters() 32-bit words that are zero before the call and zero
@@ -212,7 +247,7 @@ int ia_attention_mfma_decode_fused(void* out, float* workspace, const void* qkv,
                                    float eps, int add_one, int n, int seq_begin, int n_seqs,
                                    int token_begin, int n_tokens, int max_kv_len, int max_pages,
                                    int nq, int nkv, int d, int page_size, int window, float scale,
-                                   int splits, int chunk, int* counters, int n_counters, hipStream_t stream);
+                                   int splits, int chunk, int sink, int* counters, int n_counters, hipStream_t stream);
 
 #ifdef __cplusplus
 }

@@ -65,7 +65,8 @@ __global__ __launch_bounds__(IA_WAVE) void attn_generic_kernel(
     const int* __restrict__ block_table, // [seqs, max_pages]
     int max_pages, int nq, int nkv, int d, int page_size, int window, float scale,
     float* __restrict__ partial,         // null: a wave walks all segments; else [n, nq, segs, dpad + 2], a wave a segment
-    int segs) {
+    int segs,
+    int sink) {                          // 1: the softmax's denominator holds one more term, exp(0): a key of score 0 without a value
     __shared__ __attribute__((aligned(16))) float stage[AG_TILE * AG_PITCH];     // keys: [key][dim]; values: [dim][key]
     __shared__ __attribute__((aligned(16))) float sp[HEADS][AG_TILE];
     extern __shared__ __attribute__((aligned(16))) float ag_rows[];       // queries, a segment's outputs, the totals: [HEADS][dpad] each
@@ -361,7 +362,7 @@ __global__ __launch_bounds__(IA_WAVE) void attn_generic_kernel(
     for (int h = 0; h < HEADS; ++h) {
         if (h >= heads) break;
         T* orow = out + ((size_t)tok * nq + h0 + h) * d;
-        const float inv = 1.0f / big_l[h];
+        const float inv = 1.0f / (sink ? big_l[h] + expf(-big_m[h]) : big_l[h]);
         for (int e = lane; e < d; e += IA_WAVE) st(orow + e, st_[h * dpad + e] * inv);
     }
 }
@@ -370,7 +371,7 @@ __global__ __launch_bounds__(IA_WAVE) void attn_generic_kernel(
 template <typename T>
 __global__ __launch_bounds__(IA_WAVE) void attn_generic_merge_kernel(
     T* __restrict__ out, const float* __restrict__ partial, const int* __restrict__ positions, int nq, int d, int dpad,
-    int window, int segs) {
+    int window, int segs, int sink) {
     const int lane = threadIdx.x;
     const int tok = blockIdx.x / nq, h = blockIdx.x - tok * nq;
     const int pos = positions[tok];
@@ -393,7 +394,7 @@ __global__ __launch_bounds__(IA_WAVE) void attn_generic_merge_kernel(
             if (e < dpad) big_o[t] = ag_merge_value(big_o[t], a, row[e], b);
         }
     }
-    const float inv = 1.0f / big_l;
+    const float inv = 1.0f / (sink ? big_l + expf(-big_m) : big_l);
     T* orow = out + ((size_t)tok * nq + h) * d;
 #pragma unroll
     for (int t = 0; t < AG_MAX_HEAD_DIM / IA_WAVE; ++t) {
@@ -419,7 +420,7 @@ extern "C" int ia_attention_generic(void* out, const void* q, const void* k_cach
                                     const int* positions, const int* token_seq, const int* block_table,
                                     int n, int max_pages, int nq, int nkv, int d, int page_size,
                                     int window, float scale, int dtype, float* workspace, int max_kv_len,
-                                    hipStream_t stream) {
+                                    int sink, hipStream_t stream) {
     IA_CHECK(n >= 0 && nq > 0 && nkv > 0 && nq % nkv == 0, "attention: bad head counts nq=%d nkv=%d (n=%d)", nq, nkv, n);
     IA_CHECK(d > 0 && d <= AG_MAX_HEAD_DIM, "attention: head_dim %d is outside 1..%d", d, AG_MAX_HEAD_DIM);
     IA_CHECK(page_size > 0 && max_pages > 0, "attention: bad page geometry page_size=%d max_pages=%d", page_size, max_pages);
@@ -442,7 +443,7 @@ extern "C" int ia_attention_generic(void* out, const void* q, const void* k_cach
     const bool vec = d % 4 == 0 && page_size % 4 == 0 &&
                      (((uintptr_t)k_cache | (uintptr_t)v_cache) % (4 * elem)) == 0;
 #define AG_ARGS(T) (T*)out, (const T*)q, (const T*)k_cache, (const T*)v_cache, positions, token_seq, block_table, max_pages, nq, nkv, \
-        d, page_size, window, scale, workspace, segs
+        d, page_size, window, scale, workspace, segs, sink
     // (a wave a segment, steps of few tokens: the operands are asked for a step ahead)
 #define AG_LAUNCH(T, V, H) do { \
         if (V && workspace != nullptr) attn_generic_kernel<T, V, H, true><<<grid, IA_WAVE, rows_bytes, stream>>>(AG_ARGS(T)); \
@@ -459,9 +460,9 @@ extern "C" int ia_attention_generic(void* out, const void* q, const void* k_cach
     IA_LAUNCH_CHECK("attention_generic");
     if (workspace != nullptr) {
         if (dtype == IA_F32)
-            attn_generic_merge_kernel<float><<<(unsigned)n * nq, IA_WAVE, 0, stream>>>((float*)out, workspace, positions, nq, d, dpad, window, segs);
+            attn_generic_merge_kernel<float><<<(unsigned)n * nq, IA_WAVE, 0, stream>>>((float*)out, workspace, positions, nq, d, dpad, window, segs, sink);
         else
-            attn_generic_merge_kernel<bf16_t><<<(unsigned)n * nq, IA_WAVE, 0, stream>>>((bf16_t*)out, workspace, positions, nq, d, dpad, window, segs);
+            attn_generic_merge_kernel<bf16_t><<<(unsigned)n * nq, IA_WAVE, 0, stream>>>((bf16_t*)out, workspace, positions, nq, d, dpad, window, segs, sink);
         IA_LAUNCH_CHECK("attention_generic_merge");
     }
     return 0;

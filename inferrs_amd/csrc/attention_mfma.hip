@@ -70,6 +70,7 @@ struct AttnParams {
     const int* slots;           // [n] cache slot of each token, or null: this layer writes no cache
     float norm_eps;
     int norm_add_one;
+    int sink;                   // 1: the softmax's denominator holds one more term, 2^(0 - m): a key of score 0 without a value
 };
 
 __device__ __forceinline__ uint4 zero4() { return make_uint4(0, 0, 0, 0); }
@@ -331,7 +332,7 @@ __device__ __forceinline__ void attn_column_block(const AttnParams& p, int cb, i
         if (!cvalid[nb]) continue;
         const size_t row = (size_t)(t0 + tq[nb]) * p.nq + head[nb];
         if (p.splits == 1) {
-            const float inv = 1.0f / lt;
+            const float inv = 1.0f / (p.sink ? lt + exp2f(-m[nb]) : lt);
             bf16_t* o = p.out + row * HD + 4 * G;
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
@@ -781,7 +782,7 @@ __global__ __launch_bounds__(4 * IA_WAVE) void attn_decode_kernel(const AttnPara
         const size_t row0 = (size_t)t0 * p.nq + kvh * g + col0;        // the block's first (token, head) row
         if (p.splits == 1) {
             if (!cvalid) return;
-            const float inv = 1.0f / lt;
+            const float inv = 1.0f / (p.sink ? lt + exp2f(-m) : lt);
             bf16_t* o = p.out + (row0 + r) * HD + 4 * G;
 #pragma unroll
             for (int db = 0; db < DB; ++db) {
@@ -822,7 +823,7 @@ __global__ __launch_bounds__(4 * IA_WAVE) void attn_decode_kernel(const AttnPara
                 total = fmaf(team_ml[(w * n_cols + col) * 2 + 1], wt, total);
             }
             if (teams == 1) {
-                const float inv = 1.0f / total;
+                const float inv = 1.0f / (p.sink ? total + exp2f(-mx) : total);
                 uint2 w;
                 w.x = pack_bf16x2(o[0] * inv, o[1] * inv);
                 w.y = pack_bf16x2(o[2] * inv, o[3] * inv);
@@ -906,7 +907,7 @@ __global__ __launch_bounds__(4 * IA_WAVE) void attn_decode_kernel(const AttnPara
             } else if (!active) {
                 continue;
             }
-            const float inv = 1.0f / total;
+            const float inv = 1.0f / (p.sink ? total + exp2f(-mx) : total);
             uint2 w;
             w.x = pack_bf16x2(o[0] * inv, o[1] * inv);
             w.y = pack_bf16x2(o[2] * inv, o[3] * inv);
@@ -1357,7 +1358,7 @@ void attn_tile_kernel(const AttnParams p) {
             if (!cvalid[nb]) continue;
             const size_t row = (size_t)(t0 + tq[nb]) * p.nq + head[nb];
             if (p.splits == 1) {
-                const float inv = 1.0f / lt;
+                const float inv = 1.0f / (p.sink ? lt + exp2f(-m[nb]) : lt);
                 bf16_t* o = p.out + row * HD + 4 * G;
 #pragma unroll
                 for (int db = 0; db < DB; ++db) {
@@ -1406,7 +1407,7 @@ static int attn_cus() {
 #define MERGE_WAVES 16
 __global__ __launch_bounds__(MERGE_WAVES * IA_WAVE) void attn_merge_kernel(
     bf16_t* __restrict__ out, const float* __restrict__ part_o, const float* __restrict__ part_ml, int splits,
-    size_t first_row) {
+    size_t first_row, int sink) {
     constexpr int PER = (HD + IA_WAVE - 1) / IA_WAVE;
     __shared__ float weight[256];
     __shared__ float red[MERGE_WAVES][PER * IA_WAVE];
@@ -1438,7 +1439,7 @@ __global__ __launch_bounds__(MERGE_WAVES * IA_WAVE) void attn_merge_kernel(
             total += ml[2 * s + 1] * w;
         }
         total = wave_sum(total);
-        if (lane == 0) s_total = total;
+        if (lane == 0) s_total = sink ? total + exp2f(-mx) : total;
     }
     __syncthreads();
     float o[PER];
@@ -1476,7 +1477,7 @@ __global__ __launch_bounds__(MERGE_WAVES * IA_WAVE) void attn_merge_kernel(
 #define MERGE_ROWS_FROM 1024
 __global__ __launch_bounds__(MERGE_ROWS_WAVES * IA_WAVE) void attn_merge_rows_kernel(
     bf16_t* __restrict__ out, const float* __restrict__ part_o, const float* __restrict__ part_ml, int splits,
-    size_t first_row, size_t n_rows) {
+    size_t first_row, size_t n_rows, int sink) {
     constexpr int PER = (HD + IA_WAVE - 1) / IA_WAVE;
     const int lane = threadIdx.x & (IA_WAVE - 1), wave = threadIdx.x / IA_WAVE;
     const size_t local = (size_t)blockIdx.x * MERGE_ROWS_WAVES + wave;
@@ -1499,7 +1500,7 @@ __global__ __launch_bounds__(MERGE_ROWS_WAVES * IA_WAVE) void attn_merge_rows_ke
             if (e < HD) o[t] = fmaf(po[(size_t)s * HD + e], w, o[t]);
         }
     }
-    const float inv = 1.0f / total;
+    const float inv = 1.0f / (sink ? total + exp2f(-mx) : total);
 #pragma unroll
     for (int t = 0; t < PER; ++t) {
         const int e = lane + t * IA_WAVE;
@@ -1553,7 +1554,7 @@ static int attention_launch(void* out, float* workspace, const void* q, const vo
                             const int* positions, int n, int seq_begin, int n_seqs, int token_begin,
                             int n_tokens, int max_q_len, int max_kv_len, int max_pages,
                             int nq, int nkv, int d, int page_size, int window, float scale,
-                            int splits, int chunk, const FusedArgs* fused, hipStream_t stream) {
+                            int splits, int chunk, int sink, const FusedArgs* fused, hipStream_t stream) {
     IA_CHECK(d == HD, "attention_mfma: built for head_dim %d, called with %d", HD, d);
     IA_CHECK(n >= 0 && n_seqs >= 0 && nq > 0 && nkv > 0 && nq % nkv == 0,
              "attention_mfma: bad sizes n=%d seqs=%d nq=%d nkv=%d", n, n_seqs, nq, nkv);
@@ -1586,6 +1587,7 @@ static int attention_launch(void* out, float* workspace, const void* q, const vo
     p.max_pages = max_pages; p.nq = nq; p.nkv = nkv; p.page = page_size; p.window = window;
     p.splits = splits; p.chunk = chunk; p.seq_begin = seq_begin; p.token_begin = token_begin;
     p.scale_log2 = scale * 1.4426950408889634f;
+    p.sink = sink ? 1 : 0;
     const long long cols = (long long)max_q_len * g;
     // Columns a wave: 16 for decode, 32 for portions of prompts.  (64 keep every loaded key and
     // value in use for twice as many products but need the registers of a whole SIMD; with 32
@@ -1648,10 +1650,10 @@ static int attention_launch(void* out, float* workspace, const void* q, const vo
         if (rows >= MERGE_ROWS_FROM && splits <= 16)
             attn_merge_rows_kernel<<<(unsigned)((rows + MERGE_ROWS_WAVES - 1) / MERGE_ROWS_WAVES), MERGE_ROWS_WAVES * IA_WAVE,
                                      0, stream>>>((bf16_t*)out, p.part_o, p.part_ml, splits, (size_t)token_begin * nq,
-                                                  (size_t)rows);
+                                                  (size_t)rows, p.sink);
         else
             attn_merge_kernel<<<(unsigned)rows, MERGE_WAVES * IA_WAVE, 0, stream>>>(
-                (bf16_t*)out, p.part_o, p.part_ml, splits, (size_t)token_begin * nq);
+                (bf16_t*)out, p.part_o, p.part_ml, splits, (size_t)token_begin * nq, p.sink);
         IA_LAUNCH_CHECK("attention_merge");
     }
     return 0;
@@ -1662,10 +1664,10 @@ extern "C" int ia_attention_mfma(void* out, float* workspace, const void* q, con
                                  const int* positions, int n, int seq_begin, int n_seqs, int token_begin,
                                  int n_tokens, int max_q_len, int max_kv_len, int max_pages,
                                  int nq, int nkv, int d, int page_size, int window, float scale,
-                                 int splits, int chunk, hipStream_t stream) {
+                                 int splits, int chunk, int sink, hipStream_t stream) {
     return attention_launch(out, workspace, q, k_cache, v_cache, block_table, cu_tokens, positions, n, seq_begin,
                             n_seqs, token_begin, n_tokens, max_q_len, max_kv_len, max_pages, nq, nkv, d, page_size,
-                            window, scale, splits, chunk, nullptr, stream);
+                            window, scale, splits, chunk, sink, nullptr, stream);
 }
 
 // Whether this head size has the fused decode form.
@@ -1682,7 +1684,7 @@ extern "C" int ia_attention_mfma_decode_fused(void* out, float* workspace, const
                                               float eps, int add_one, int n, int seq_begin, int n_seqs,
                                               int token_begin, int n_tokens, int max_kv_len, int max_pages,
                                               int nq, int nkv, int d, int page_size, int window, float scale,
-                                              int splits, int chunk, int* counters, int n_counters,
+                                              int splits, int chunk, int sink, int* counters, int n_counters,
                                               hipStream_t stream) {
     IA_CHECK(qkv != nullptr && (q_norm_w == nullptr) == (k_norm_w == nullptr) && (cos_t == nullptr) == (sin_t == nullptr),
              "attention_mfma_decode_fused: qkv is needed; norm weights and angle tables come in pairs");
@@ -1692,5 +1694,5 @@ extern "C" int ia_attention_mfma_decode_fused(void* out, float* workspace, const
     const FusedArgs fused = {qkv, q_norm_w, k_norm_w, cos_t, sin_t, slots, eps, add_one, counters, n_counters};
     return attention_launch(out, workspace, nullptr, k_cache, v_cache, block_table, cu_tokens, positions, n, seq_begin,
                             n_seqs, token_begin, n_tokens, 1, max_kv_len, max_pages, nq, nkv, d, page_size,
-                            window, scale, splits, chunk, &fused, stream);
+                            window, scale, splits, chunk, sink, &fused, stream);
 }

@@ -51,6 +51,7 @@ class StepContext:
     stream: Optional[torch.Tensor] = None   # set by a block around a part that may add its output to it itself
     stream_norm: Any = None                 # and the norm part that will read the stream next
     partial_sums: bool = False              # set by a block whose norms take a part's last product split along k
+    pass_input: Any = None                  # set by the model before a stop that begins a pass of a looped range: (rows or None, vector); the block takes it
     _tables: Dict[Any, Any] = field(default_factory=dict)
 
     @property

@@ -8,7 +8,7 @@ from typing import Dict, Optional
 import torch
 
 from .. import ops
-from ..config.spec import ModelSpec
+from ..config.spec import ModelSpec, SpecError
 from ..parts.base import block_class, part_class
 from ..parts.linear import Linear
 from .batch import StepContext
@@ -46,6 +46,10 @@ class DecoderModel:
         for layer in spec.layers:
             cls = block_class(layer)
             self.blocks.append(cls(layer, take(cls.tensors(layer)), dtype, device))
+        self.pass_input = None
+        if spec.pass_input is not None:
+            pass_cls = part_class("pass_input", spec.pass_input)
+            self.pass_input = pass_cls(spec.pass_input, take(pass_cls.tensors(spec.pass_input)), dtype, device)
         self.final_norm = None
         if spec.final_norm is not None:
             self.final_norm = part_class("norm", spec.final_norm)(
@@ -54,13 +58,10 @@ class DecoderModel:
     @property
     def graph_safe(self) -> bool:
         """Whether every part allows a decode step to be captured and replayed."""
-        parts = [self.embedding, self.head, self.final_norm]
-        for b in self.blocks:
-            parts += list(b.parts())
-        return all(getattr(p, "graph_safe", False) for p in parts if p is not None)
+        return all(getattr(p, "graph_safe", False) for p in self.all_parts())
 
     def all_parts(self):
-        parts = [self.embedding, self.head, self.final_norm]
+        parts = [self.embedding, self.head, self.final_norm, self.pass_input]
         for b in self.blocks:
             parts += list(b.parts())
         return [p for p in parts if p is not None]
@@ -87,7 +88,7 @@ class DecoderModel:
     def forward(self, ctx: StepContext, storage) -> torch.Tensor:
         """Runs the step's tokens through every stop of the schedule (which appends to the
         caches) and returns float32 logits `[n_want, vocab]`."""
-        x = self.embedding.forward(ctx)
+        x = first_rows = self.embedding.forward(ctx)
         first = self.blocks[self.spec.schedule[0].layer]
         if hasattr(first, "enter"):                  # an arrangement whose stream is not the embedding's rows
             x = first.enter(ctx, x)
@@ -98,7 +99,12 @@ class DecoderModel:
                 cache = cache.reader()
             after = self.spec.schedule[stop + 1].layer if stop + 1 < len(self.spec.schedule) else None
             next_norm = self.blocks[after].first_norm if after is not None else None
+            if e.pass_index is not None and self.pass_input is not None:
+                ctx.pass_input = self.pass_input.inputs(first_rows, e.pass_index)
             x, pending = self.blocks[e.layer].forward(ctx, x, pending, cache, next_norm)
+            if ctx.pass_input is not None:
+                raise SpecError(f"the arrangement {self.spec.layers[e.layer].arrangement!r} does not take what enters the "
+                                "stream before a pass of a looped range")
         n_want = ctx.want_rows.numel()
         if n_want == 0:
             return torch.empty((0, self.spec.vocab_size), dtype=torch.float32, device=x.device)
@@ -123,12 +129,7 @@ class DecoderModel:
             nonlocal total
             if t is not None and t.data_ptr() not in seen:
                 seen.add(t.data_ptr()); total += t.numel() * t.element_size()
-        parts = [self.embedding, self.head, self.final_norm]
-        for b in self.blocks:
-            parts += list(b.parts())
-        for part in parts:
-            if part is None:
-                continue
+        for part in self.all_parts():
             for v in vars(part).values():
                 if isinstance(v, torch.Tensor):
                     add(v)

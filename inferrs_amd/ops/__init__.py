@@ -360,12 +360,13 @@ def _check_cache(k_cache: torch.Tensor, v_cache: torch.Tensor, nkv: int, page_si
 def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor,
                       positions: torch.Tensor, token_seq: torch.Tensor, block_table: torch.Tensor,
                       *, window: Optional[int], scale: float, max_kv_len: Optional[int] = None,
-                      split: Optional[bool] = None) -> torch.Tensor:
+                      split: Optional[bool] = None, sink: bool = False) -> torch.Tensor:
     """q [n, nq, d] against the paged cache; token i sees the keys at positions <= positions[i]
     (and > positions[i] - window) of row token_seq[i] of the table.  Any head size up to 512, any
     page size, 32-bit or bfloat16 storage, all arithmetic in 32-bit.  `max_kv_len`: an upper bound of
     positions + 1 (default: what the table can hold).  Steps of few tokens run a wave a segment of 512 keys
-    and a merge kernel (`split`; None: the kernel's own rule); the bits are the same either way."""
+    and a merge kernel (`split`; None: the kernel's own rule); the bits are the same either way.
+    `sink`: the softmax's denominator holds one more term, exp(0): a key of score 0 that has no value."""
     _dev(q, k_cache, v_cache, positions, token_seq, block_table)
     _i32(positions, "positions"); _i32(token_seq, "token_seq"); _i32(block_table, "block_table")
     n, nq, d = q.shape
@@ -384,7 +385,7 @@ def attention_generic(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Ten
     _check(lib.ia_attention_generic(
         _p(out), _p(q), _p(k_cache), _p(v_cache), _p(positions), _p(token_seq), _p(block_table), n,
         block_table.shape[1], nq, nkv, d, page_size, int(window or 0), ctypes.c_float(scale), _dt(q),
-        _p(ws), max_kv_len, _stream()))
+        _p(ws), max_kv_len, int(bool(sink)), _stream()))
     return out
 
 
@@ -461,7 +462,7 @@ def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
                    cu_tokens: torch.Tensor, block_table: torch.Tensor, *, max_q_len: int, max_kv_len: int,
                    window: Optional[int], scale: float, splits: Optional[int] = None,
                    seqs: Optional[Tuple[int, int]] = None, tokens: Optional[Tuple[int, int]] = None,
-                   out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                   out: Optional[torch.Tensor] = None, sink: bool = False) -> torch.Tensor:
     """The matrix-core kernel: bfloat16, head sizes in steps of 16 up to 256, page sizes in steps
     of 16.  Request s owns tokens cu_tokens[s]..cu_tokens[s+1] at consecutive positions.  `seqs` =
     (first, count) and `tokens` = (first, count) restrict the call to a run of requests and their
@@ -501,7 +502,7 @@ def attention_mfma(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor
     _check(lib.ia_attention_mfma(
         _p(out), _p(ws), _p(q), _p(k_cache), _p(v_cache), _p(block_table), _p(cu_tokens), _p(positions),
         n, seq_begin, n_seqs, token_begin, n_tokens, max_q_len, max_kv_len, block_table.shape[1], nq, nkv, d,
-        page_size, int(window or 0), ctypes.c_float(scale), splits, chunk, _stream()), target)
+        page_size, int(window or 0), ctypes.c_float(scale), splits, chunk, int(bool(sink)), _stream()), target)
     return out
 
 
@@ -542,7 +543,8 @@ def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
                            k_norm_w: Optional[torch.Tensor], eps: float, add_one: bool,
                            cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], max_kv_len: int,
                            window: Optional[int], scale: float, splits: Optional[int] = None,
-                           seqs: Optional[Tuple[int, int]] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+                           seqs: Optional[Tuple[int, int]] = None, out: Optional[torch.Tensor] = None,
+                           sink: bool = False) -> torch.Tensor:
     """Decode steps (one token a request) in one kernel: per-head norm of q and k, rotation, the write
     of the new key and value at `slots` (None: the cache is only read) and the attention over the pages.
     `qkv` [n, (nq + 2 nkv) * d] is the projections' output; request s owns token s.  Returns [n, nq, d]."""
@@ -594,7 +596,7 @@ def attention_decode_fused(qkv: torch.Tensor, k_cache: torch.Tensor, v_cache: to
         _p(out), _p(ws), _p(qkv), _p(k_cache), _p(v_cache), _p(block_table), _p(cu_tokens), _p(positions), _p(slots),
         _p(q_norm_w), _p(k_norm_w), _p(cos), _p(sin), ctypes.c_float(eps), int(add_one), n, seq_begin, n_seqs,
         seq_begin, n_seqs, max_kv_len, block_table.shape[1], nq, nkv, d, page_size, int(window or 0),
-        ctypes.c_float(scale), splits, chunk, _p(counters), counters.numel() if counters is not None else 0,
+        ctypes.c_float(scale), splits, chunk, int(bool(sink)), _p(counters), counters.numel() if counters is not None else 0,
         _stream()), target)
     return out
 
@@ -1184,3 +1186,6 @@ def gated_silu_linear(x, w_gate_up: torch.Tensor) -> torch.Tensor:
 # ---- several residual streams, latent attention, gated recurrence, routed experts -----------------
 from .mix import (conv_step, experts_forward, head_product, latent_prep, rglru_scan, route, softcap,   # noqa: E402
                   streams_open, streams_step)
+from .state import (activation, conv_act_step, exp_gates, group_norm_gate, linear_scan, sandwich_step,   # noqa: E402
+                    step_gates)
+from . import state                                                                                    # noqa: E402

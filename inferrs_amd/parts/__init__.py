@@ -1,7 +1,8 @@
-from .base import (BlockBase, Embedding, FeedForward, FixedState, Head, Mixer, Norm, PagedKV, Part, Position,
+from .base import (BlockBase, Embedding, FeedForward, FixedState, Head, Mixer, Norm, PagedAndState, PagedKV, Part, Position,
                    block_class, part_class, register_block, register_embedding, register_ffn, register_head,
-                   register_mixer, register_norm, register_position)
-from . import norm, position, mlp, attention, io, block, latent_attention, recurrence, experts, streams   # registers the built-in parts
+                   register_mixer, register_norm, register_pass_input, register_position)
+from . import (norm, position, mlp, attention, io, block, latent_attention, recurrence, experts, streams,   # registers the built-in parts
+               sandwich, matrix_state)
 from .assemble import generated_tensors, layer_tensors, model_tensors
 from .block import Block
 from .linear import Linear

@@ -22,6 +22,8 @@ def model_tensors(spec: ModelSpec) -> Tuple[Dict[str, TensorSpec], Set[str]]:
         expected[spec.final_norm_name] = ts
     head = part_class("head", spec.head)
     expected.update(head.tensors(spec.head))
+    if getattr(spec, "pass_input", None) is not None:
+        expected.update(part_class("pass_input", spec.pass_input).tensors(spec.pass_input))
     optional: Set[str] = set(head.optional(spec.head)) if hasattr(head, "optional") else set()
     return expected, optional
 

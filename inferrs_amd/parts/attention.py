@@ -6,6 +6,11 @@ position; append of k and v to the cache; scores (q.k)/sqrt(d) against keys at p
 <= the query's (and inside the window, when one is set); softmax; weighted sum of values;
 output projection.  q head h reads kv head h // (n_heads / n_kv_heads)
 (`attention_utils.rs:38-49`).
+
+Options of the spec beyond the reference's layer: biases, a window, a sink in the softmax (`sink`: the denominator
+holds one more term, exp(0)), values that are the keys as projected, before norm and rotation (`values_from_keys`: no
+value projection is loaded; the key projection's rows stand twice in the fused product, so the kernels that take
+[q | k | v] serve unchanged), and other names for the tensors in the file (`names`).
 """
 from __future__ import annotations
 
@@ -28,6 +33,14 @@ class Attention(Mixer):
 
     @classmethod
     def tensors(cls, spec: AttentionSpec) -> Dict[str, TensorSpec]:
+        named = dict(spec.names or ())
+        t = cls._tensors(spec)
+        if spec.values_from_keys:
+            t = {k: v for k, v in t.items() if not k.startswith("v_proj.")}
+        return {named.get(k, k): v for k, v in t.items()}
+
+    @classmethod
+    def _tensors(cls, spec: AttentionSpec) -> Dict[str, TensorSpec]:
         q_out, kv_out = spec.n_heads * spec.head_dim, spec.n_kv_heads * spec.head_dim
         t = {
             "q_proj.weight": TensorSpec((q_out, spec.hidden)),
@@ -65,6 +78,12 @@ class Attention(Mixer):
         if spec.qk_norm is not None and spec.qk_norm.size != spec.head_dim:
             raise SpecError("attention: qk_norm must span head_dim")
         self.spec = spec
+        named = dict(spec.names or ())
+        tensors = {k: tensors[named.get(k, k)] for k in self._tensors(spec) if named.get(k, k) in tensors}
+        if spec.values_from_keys:
+            tensors["v_proj.weight"] = tensors["k_proj.weight"]
+            if spec.qkv_bias:
+                tensors["v_proj.bias"] = tensors["k_proj.bias"]
         self.qkv = Linear([tensors["q_proj.weight"], tensors["k_proj.weight"], tensors["v_proj.weight"]], dtype, device,
                           [tensors["q_proj.bias"], tensors["k_proj.bias"], tensors["v_proj.bias"]] if spec.qkv_bias else None)
         self.o = Linear([tensors["o_proj.weight"]], dtype, device, [tensors["o_proj.bias"]] if spec.o_bias else None)
@@ -121,7 +140,7 @@ class Attention(Mixer):
                 qkv, cache.k, cache.v, ctx.positions, ctx.cu_tokens, group.block_table, nq=s.n_heads,
                 nkv=s.n_kv_heads, d=s.head_dim, slots=group.slots if cache.writable else None,
                 q_norm_w=self.q_norm_w, k_norm_w=self.k_norm_w, eps=self.norm_eps, add_one=self.norm_add_one,
-                cos=cos, sin=sin, max_kv_len=ctx.max_kv_len, window=s.window, scale=s.softmax_scale)
+                cos=cos, sin=sin, max_kv_len=ctx.max_kv_len, window=s.window, scale=s.softmax_scale, sink=s.sink)
             return self._project(ctx, a.view(a.shape[0], s.n_heads * s.head_dim))
         q = ops.qk_rope_kv(
             qkv, s.n_heads, s.n_kv_heads, s.head_dim,
@@ -130,7 +149,7 @@ class Attention(Mixer):
             k_cache=cache.k, v_cache=cache.v, slots=group.slots if cache.writable else None,
             page_size=group.page_size)
         if ops.attention_mfma_fits(q.dtype, s.head_dim, group.page_size):
-            common = dict(window=s.window, scale=s.softmax_scale)
+            common = dict(window=s.window, scale=s.softmax_scale, sink=s.sink)
             if 0 < ctx.n_single < ctx.n_seqs:
                 # single tokens (decode) and portions of prompts want different launches: the first
                 # split their long key ranges between waves, the second have columns enough
@@ -146,5 +165,5 @@ class Attention(Mixer):
                                        max_q_len=ctx.max_q_len, max_kv_len=ctx.max_kv_len, **common)
         else:
             a = ops.attention_generic(q, cache.k, cache.v, ctx.positions, ctx.token_seq, group.block_table,
-                                      window=s.window, scale=s.softmax_scale, max_kv_len=ctx.max_kv_len)
+                                      window=s.window, scale=s.softmax_scale, max_kv_len=ctx.max_kv_len, sink=s.sink)
         return self._project(ctx, a.view(a.shape[0], s.n_heads * s.head_dim))

@@ -77,10 +77,18 @@ class FixedState:
         return n * torch.empty((), dtype=self.dtype).element_size()
 
 
+@dataclass(frozen=True)
+class PagedAndState:
+    """Both: pages of keys and values and a state of fixed size (a mixer of two branches side by side, one that
+    attends to cached keys and one that carries a state).  The mixer's `LayerCache` holds `k`, `v` and `state`."""
+    paged: PagedKV
+    state: FixedState
+
+
 # ---- registries -----------------------------------------------------------------------------
 
 _TABLES: Dict[str, Dict[str, type]] = {"mixer": {}, "ffn": {}, "norm": {}, "position": {}, "block": {},
-                                       "embedding": {}, "head": {}}
+                                       "embedding": {}, "head": {}, "pass_input": {}}
 
 
 def _register(table: str, kind: str) -> Callable[[type], type]:
@@ -121,6 +129,12 @@ def register_head(kind: str):
     return _register("head", kind)
 
 
+def register_pass_input(kind: str):
+    """What enters the stream before a pass over a looped range of layers: a class with `tensors(spec)`,
+    `__init__(spec, tensors, dtype, device)` and `inputs(first_rows, t) -> (rows or None, vector or None)`."""
+    return _register("pass_input", kind)
+
+
 def block_class(layer_spec: Any) -> type:
     try:
         return _TABLES["block"][layer_spec.arrangement]
@@ -159,7 +173,7 @@ class Part:
 class Mixer(Part):
     @classmethod
     def cache_need(cls, spec):
-        """`PagedKV`, `FixedState` or None."""
+        """`PagedKV`, `FixedState`, `PagedAndState` or None."""
         return None
 
     def forward(self, ctx, h: torch.Tensor, cache) -> torch.Tensor:

@@ -10,7 +10,7 @@ import torch
 
 from .. import ops
 from ..weights.loader import TensorSpec
-from .base import Embedding, Head, register_embedding, register_head
+from .base import Embedding, Head, Part, register_embedding, register_head, register_pass_input
 from .linear import Linear, to_compute
 
 
@@ -76,3 +76,24 @@ class CappedHead(LinearHead):
         if self.spec.cap is not None:
             ops.softcap(logits, float(self.spec.cap))
         return logits
+
+
+@register_pass_input("pass_input")
+class PassInput(Part):
+    """What enters the stream before pass t over a looped range of layers: row t of a [times, hidden] tensor (kept in
+    32-bit) and, before every pass but the first, the embedding's rows once more.  The block that runs first in the pass
+    adds them."""
+    graph_safe = True
+
+    @classmethod
+    def tensors(cls, spec) -> Dict[str, TensorSpec]:
+        return {spec.name: TensorSpec((spec.times, spec.hidden), "matrix")}
+
+    def __init__(self, spec, tensors: Dict[str, torch.Tensor], dtype, device):
+        self.spec = spec
+        self.steps = tensors[spec.name].to(device=device, dtype=torch.float32).contiguous()
+
+    def inputs(self, first_rows: torch.Tensor, t: int):
+        if not (0 <= t < self.spec.times):
+            raise ValueError(f"pass {t} of a range that runs {self.spec.times} times")
+        return (first_rows if self.spec.readd_embedding and t > 0 else None), self.steps[t]

@@ -8,7 +8,7 @@ from typing import Dict
 import torch
 
 from .. import ops
-from ..config.spec import GatedMlpSpec, SpecError
+from ..config.spec import DenseMlpSpec, GatedMlpSpec, SpecError
 from ..weights.loader import TensorSpec
 from .base import FeedForward, register_ffn
 from .linear import Linear
@@ -53,3 +53,26 @@ class GatedMlp(FeedForward):
             if split is not None:
                 return split
         return self.down(act)
+
+
+@register_ffn("dense_mlp")
+class DenseMlp(FeedForward):
+    """down( act(up(x)) ) without a gate: tensors "up" and "down"."""
+    graph_safe = True
+    ACTIVATIONS = {"silu": ops.state.ACT_SILU, "gelu_tanh": ops.state.ACT_GELU_TANH, "gelu": ops.state.ACT_GELU}
+
+    @classmethod
+    def tensors(cls, spec: DenseMlpSpec) -> Dict[str, TensorSpec]:
+        return {"up": TensorSpec((spec.intermediate, spec.hidden)), "down": TensorSpec((spec.hidden, spec.intermediate))}
+
+    def __init__(self, spec: DenseMlpSpec, tensors: Dict[str, torch.Tensor], dtype, device):
+        if spec.activation not in self.ACTIVATIONS:
+            raise SpecError(f"dense_mlp: activation {spec.activation!r} has no kernel (known: {sorted(self.ACTIVATIONS)})")
+        self.spec = spec
+        self.up = Linear([tensors["up"]], dtype, device)
+        self.down = Linear([tensors["down"]], dtype, device)
+
+    def forward(self, ctx, h):
+        if hasattr(h, "materialize"):
+            h = h.materialize()
+        return self.down(ops.activation(self.up(h), self.ACTIVATIONS[self.spec.activation]))
