@@ -67,7 +67,7 @@ def rotate_halves(x: torch.Tensor, positions: torch.Tensor, base: float, dims: i
 def sink_window_attention(h: torch.Tensor, w: T, p: str, m: dict, eps: float) -> torch.Tensor:
     n = h.shape[0]
     H, G, d = int(m["heads"]), int(m["kv_heads"]), int(m["dim"])
-    window, scale = int(m["mask"]["size"]), float(m["scale"])
+    window, scale = int((m.get("mask") or {}).get("size", n + 1)), float(m["scale"])      # no mask: every earlier key
     q = (h @ w[p + "q"].T + w[p + "q.b"]).view(n, H, d)
     k = (h @ w[p + "k"].T + w[p + "k.b"]).view(n, G, d)
     v = k                                             # the values: the keys before norm and rotation
