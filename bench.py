@@ -18,9 +18,10 @@ choice): `mixed16` is 16 requests with prompts of 128 to 4,096 random tokens in 
 `--decode-tokens` tokens.  Its JSON line gives tokens a second over the whole run, the prompts' and the
 decoded tokens' rates apart, and the time to a request's first token.
 
-    python bench.py --design buketar [--design-shapes 1k,2k,4k]
+    python bench.py --design buketar|lofudra [--design-shapes 1k,2k,4k]
 
-measures the Buketar design (latent attention, gated recurrences, routed experts, residual streams) at a few layer
+measures the Buketar design (latent attention, gated recurrences, routed experts, residual streams) or the Lofudra
+design (windowed sink attention beside retention, matrix memory, state space, norms on both sides) at a few layer
 sizes beside the dense decoder at equal width, layers and feed-forward products a token: prompts of `--prefill-tokens`
 tokens, decode steps at `--batch` and at batch 1 through the serving loop, and every kernel's time in one prompt and one
 decode step of both.  One JSON line; the default record above is not touched by it.
@@ -386,20 +387,61 @@ LIKE_KERNEL = {"streams_step": "add_rmsnorm", "latent_prep": "qk_rope_kv", "head
                "conv_step": "add_rmsnorm", "route": "rmsnorm", "route_plan": "rmsnorm", "softcap": "rmsnorm"}
 
 
+# ---- the Lofudra design beside the dense decoder at equal size (`--design lofudra`) ---------------------------
+# Layer sizes in the range of real models of its mixers: a state space of 2 x width inner features in heads of 64 with a
+# state of 128; windowed attention in heads of 128 (a window of 1,024) beside a retention of as many heads with keys of
+# 64 and values of 128; a matrix memory in heads of 128 x 256; a feed-forward of 4 x width.  The dense twin has the same
+# width and number of layers, as many attention heads of size 128 as fill the width, and a gated feed-forward of the
+# same products a token (2/3 of the size, three matrices for two).
+def lofudra_shape(width: int, layers: int, vocab: int = 32768):
+    heads = width // 128
+    ssm = {"type": "mamba2", "mixer": {"heads": 2 * width // 64, "vdim": 64, "state": 128, "groups": 1, "conv": 4, "norm_groups": 1}}
+    par = {"type": "parallel",
+           "mixer": {"left": {"heads": heads, "kv_heads": max(1, heads // 4), "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                              "mask": {"size": 1024}, "rot": {"base": 500000.0, "dims": 128}},
+                     "right": {"heads": heads, "dim": 64, "vdim": 128, "decay": [1.0 - 2.0 ** (-5 - 5 * i / max(heads - 1, 1)) for i in range(heads)]},
+                     "left_scale": 1.0, "right_scale": 1.0}}
+    mem = {"type": "mlstm", "mixer": {"heads": max(1, width // 256), "dim": 128, "vdim": 256, "gate_cap": 15.0}}
+    pattern = [ssm, par, mem]
+    return {"architecture": "Lofudra", "vocab": vocab, "width": width, "norm": {"eps": 1e-6},
+            "layers": [dict(pattern[i % 3], mlp={"kind": "dense", "ff": 4 * width}) for i in range(layers)]}
+
+
+LOFUDRA_SHAPES = {"1k": dict(width=1024, layers=12), "2k": dict(width=2048, layers=12), "4k": dict(width=4096, layers=6)}
+
+
+def lofudra_twin(b: dict, vocab: int = 32768) -> dict:
+    return dict(QWEN3_8B, vocab_size=vocab, hidden_size=b["width"], intermediate_size=8 * b["width"] // 3 // 128 * 128,
+                num_hidden_layers=b["layers"], num_attention_heads=b["width"] // 128, num_key_value_heads=max(1, b["width"] // 512),
+                tie_word_embeddings=False)
+
+
+LOFUDRA_LIKE_KERNEL = {"sandwich_step": "add_rmsnorm", "activation": "gate_mul", "conv_act_step": "add_rmsnorm",
+                       "group_norm_gate": "rmsnorm", "exp_gates": "rmsnorm", "step_gates": "rmsnorm",
+                       "linear_scan": "attention_mfma", "linear_scan_chunked": "attention_mfma"}
+
+
 def design_main(args) -> int:
-    """Prefill and decode throughput of the Buketar design at a few layer sizes beside the dense decoder at equal
+    """Prefill and decode throughput of a design at a few layer sizes beside the dense decoder at equal
     size (random weights), and the time of every kernel of one prefill and one decode step of both."""
     import torch
     from inferrs_amd.config import Qwen3Config
     from inferrs_amd.config.buketar import BuketarConfig
+    from inferrs_amd.config.lofudra import LofudraConfig
     from inferrs_amd.engine import Engine
     batch, context, prompt = args.batch, min(args.context, 2048), args.prefill_tokens
     records = {}
-    for name in (args.design_shapes.split(",") if args.design_shapes else sorted(BUKETAR_SHAPES)):
-        b = BUKETAR_SHAPES[name]
-        raw_new, raw_old = buketar_shape(**b), dense_twin(b)
+    if args.design == "lofudra":
+        shapes, shape_of, twin_of, config_cls, like = LOFUDRA_SHAPES, lofudra_shape, lofudra_twin, LofudraConfig, LOFUDRA_LIKE_KERNEL
+        title, beside = "Lofudra", "Qwen3 dense at equal width, layers and feed-forward products a token"
+    else:
+        shapes, shape_of, twin_of, config_cls, like = BUKETAR_SHAPES, buketar_shape, dense_twin, BuketarConfig, LIKE_KERNEL
+        title, beside = "Buketar", "Qwen3 dense at equal width, layers and feed-forward products a token"
+    for name in (args.design_shapes.split(",") if args.design_shapes else sorted(shapes)):
+        b = shapes[name]
+        raw_new, raw_old = shape_of(**b), twin_of(b)
         rec = {}
-        for label, config, vocab in (("buketar", BuketarConfig.from_dict(raw_new), raw_new["vocab"]),
+        for label, config, vocab in ((args.design, config_cls.from_dict(raw_new), raw_new["vocab"]),
                                      ("dense", Qwen3Config.from_dict(raw_old), raw_old["vocab_size"])):
             pages = batch * (-(-context // PAGE) + 1) + -(-prompt // PAGE) + 8
             note(f"{name} {label}: random weights, {pages} pages")
@@ -418,9 +460,8 @@ def design_main(args) -> int:
             del engine
             torch.cuda.empty_cache()
         records[name] = rec
-    print(json.dumps({"metric": "design_throughput", "design": "Buketar", "beside": "Qwen3 dense at equal width, layers and "
-                      "feed-forward products a token", "dtype": args.dtype, "data": "synthetic", "batch": batch, "context": context,
-                      "prefill_tokens": prompt, "steps": args.steps, "warmup": args.warmup, "like_kernel": LIKE_KERNEL,
+    print(json.dumps({"metric": "design_throughput", "design": title, "beside": beside, "dtype": args.dtype, "data": "synthetic", "batch": batch, "context": context,
+                      "prefill_tokens": prompt, "steps": args.steps, "warmup": args.warmup, "like_kernel": like,
                       "shapes": records}))
     return 0
 
@@ -457,7 +498,7 @@ def main() -> int:
                     help="workloads: cut prompt portions so that a step's tokens are a multiple of this (0: off)")
     ap.add_argument("--decode-run", type=int, default=8,
                     help="decode steps that the serving loop queues on the GPU at once (1: one at a time)")
-    ap.add_argument("--design", default=None, choices=["buketar"],
+    ap.add_argument("--design", default=None, choices=["buketar", "lofudra"],
                     help="instead of the headline: prefill and decode throughput of this design at a few layer sizes "
                          "beside the dense decoder at equal size, with every kernel's time")
     ap.add_argument("--design-shapes", default=None, help="with --design: the sizes to run, with commas (default: all)")

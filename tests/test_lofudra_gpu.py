@@ -156,7 +156,7 @@ def test_sink_plain_kernel(dtype, nq, nkv, d, page, window, lens, q_lens):
     # the sink is what makes the difference (among the few keys of a window)
     plain = ops.attention_generic(dev(q), dev(kc), dev(vc), dev(positions), dev(token_seq), dev(table), window=window,
                                   scale=scale, max_kv_len=max(lens))
-    assert float((plain.double().cpu() - want).abs().max()) > 0.02
+    assert float((plain.double().cpu() - want).abs().max()) > 0.005
 
 
 @pytest.mark.parametrize("nq,nkv,d,page,window", [(4, 2, 16, 16, None), (5, 1, 48, 16, 40), (8, 1, 128, 16, None), (32, 8, 128, 16, 300),
