@@ -207,18 +207,22 @@ int ia_conv_act_step(void* out, const void* x, const void* taps, const void* bia
 int ia_exp_gates(float* log_a, float* b, float* floor_, float* state, long long row_floats, long long m_off,
                  const void* proj, long long p_ld, int i_off, int f_off, const float* bias_i,
                  const float* bias_f, float cap, const int* cu_tokens, const int* state_slots, int H,
-                 int n_seqs, int dtype, hipStream_t stream);
+                 int n_seqs, int max_q_len, int dtype, hipStream_t stream);
 int ia_step_gates(float* log_a, float* b, const void* proj, long long p_ld, int dt_off, const float* dt_bias,
                   const float* a_log, int n, int H, int dtype, hipStream_t stream);
 // S <- a S + b k v^T, o = S^T q (+ skip v); `den` not null: one more column of S whose value is always 1.
 // log_a: [n][H] logarithms of the decays (a_per_token 1) or the decays themselves, [H] (a_per_token 0).
+// chunk > 0: portions run in chunks of that many tokens side by side (workspace: ia_linear_scan_workspace floats; max_q_len:
+// an upper bound of a request's tokens); the results differ from the walk (chunk 0) by rounding.
 int ia_linear_scan(float* out, float* den, float* state, long long row_floats, long long s_off,
                    const void* q, long long q_ld, int q_off, int q_heads,
                    const void* k, long long k_ld, int k_off, int k_heads,
                    const void* v, long long v_ld, int v_off,
                    const float* log_a, int a_per_token, const float* b, const float* skip,
                    const int* cu_tokens, const int* state_slots, int n_seqs, int H, int dim, int vdim,
-                   float q_scale, float k_scale, int dtype, hipStream_t stream);
+                   float q_scale, float k_scale, int chunk, int max_q_len, float* workspace, int dtype,
+                   hipStream_t stream);
+long long ia_linear_scan_workspace(int n_seqs, int max_q_len, int chunk, int H, int dim, int vdim, int normaliser);
 // [o / (max(|den|, floor) + 1e-6)] [* act(gate)] -> RMS norm in groups of `group` features [* w] [* act(gate)]; act: 1 SiLU, 4 sigmoid
 int ia_group_norm_gate(void* out, const float* o, const float* den, const float* floor_, int head,
                        const void* gate, long long g_ld, int g_off, int act, int gate_first, const float* w,

@@ -124,14 +124,80 @@ __global__ void exp_gates_kernel(float* __restrict__ log_a, float* __restrict__ 
     *mp = m;
 }
 
+// The same for long portions: a block a (request, head); thread i owns a run of neighbouring tokens.  A token's step
+// m -> max(m + f, i) is the pair (f, i); two steps in a row are the pair (f1 + f2, max(i1 + f2, i2)), so the runs are
+// folded first, the block's threads' pairs are folded in order by one thread, and every thread then walks its run from
+// the maximum it starts with.  The sums of f inside a pair matter only while they are small (beyond that the second
+// entry wins the maximum), so the result differs from the walk above by rounding only.
+#define EG_THREADS 256
+template <typename T>
+__global__ __launch_bounds__(EG_THREADS) void exp_gates_block_kernel(
+    float* __restrict__ log_a, float* __restrict__ b, float* __restrict__ floor_, float* __restrict__ state,
+    long long row_floats, long long m_off, const T* __restrict__ proj, long long p_ld, int i_off, int f_off,
+    const float* __restrict__ bias_i, const float* __restrict__ bias_f, float cap, const int* __restrict__ cu_tokens,
+    const int* __restrict__ state_slots, int H) {
+    __shared__ float sf[EG_THREADS], si[EG_THREADS], start[EG_THREADS];
+    const int seq = blockIdx.x / H, h = blockIdx.x - seq * H;
+    const int first = cu_tokens[seq], last = cu_tokens[seq + 1];
+    const int per = (last - first + EG_THREADS - 1) / EG_THREADS;
+    const int lo = first + threadIdx.x * per < last ? first + threadIdx.x * per : last;
+    const int hi = lo + per < last ? lo + per : last;
+    float* mp = state + (long long)state_slots[seq] * row_floats + m_off + h;
+    const float bi = bias_i[h], bf = bias_f[h];
+    // the run's gates (parked where the results go) and its pair
+    float sum_f = 0.f, top = -INFINITY;
+    for (int t = lo; t < hi; ++t) {
+        const float gi = cap * tanhf((ld(proj + (long long)t * p_ld + i_off + h) + bi) / cap);
+        const float zf = cap * tanhf((ld(proj + (long long)t * p_ld + f_off + h) + bf) / cap);
+        const float gf = -ls_softplus(-zf);
+        log_a[(long long)t * H + h] = gf;
+        b[(long long)t * H + h] = gi;
+        sum_f += gf;
+        top = fmaxf(top + gf, gi);
+    }
+    sf[threadIdx.x] = sum_f; si[threadIdx.x] = top;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        float m = *mp;
+        for (int i = 0; i < EG_THREADS; ++i) {
+            start[i] = m;
+            m = fmaxf(m + sf[i], si[i]);                         // (an empty run is the pair (0, -inf): m stays)
+        }
+        *mp = m;
+    }
+    __syncthreads();
+    float m = start[threadIdx.x];
+    for (int t = lo; t < hi; ++t) {
+        const float gf = log_a[(long long)t * H + h], gi = b[(long long)t * H + h];
+        const float m_new = fmaxf(gf + m, gi);
+        log_a[(long long)t * H + h] = gf + m - m_new;
+        b[(long long)t * H + h] = expf(gi - m_new);
+        floor_[(long long)t * H + h] = expf(-m_new);
+        m = m_new;
+    }
+}
+
+// max_q_len: an upper bound of the tokens a request brings (steps with long portions take a block a (request, head))
 extern "C" int ia_exp_gates(float* log_a, float* b, float* floor_, float* state, long long row_floats, long long m_off,
                             const void* proj, long long p_ld, int i_off, int f_off, const float* bias_i,
                             const float* bias_f, float cap, const int* cu_tokens, const int* state_slots, int H,
-                            int n_seqs, int dtype, hipStream_t stream) {
+                            int n_seqs, int max_q_len, int dtype, hipStream_t stream) {
     IA_CHECK(H > 0 && n_seqs >= 0 && cap > 0.f && i_off >= 0 && f_off >= 0 && i_off + H <= p_ld && f_off + H <= p_ld,
              "exp_gates: bad sizes heads=%d cap=%g", H, (double)cap);
     IA_CHECK(m_off >= 0 && m_off + H <= row_floats, "exp_gates: the maxima do not fit the state row");
     if (n_seqs == 0) return 0;
+    if (max_q_len > 32) {
+        if (dtype == IA_F32)
+            exp_gates_block_kernel<float><<<(unsigned)(n_seqs * H), EG_THREADS, 0, stream>>>(
+                log_a, b, floor_, state, row_floats, m_off, (const float*)proj, p_ld, i_off, f_off, bias_i, bias_f, cap, cu_tokens,
+                state_slots, H);
+        else
+            exp_gates_block_kernel<bf16_t><<<(unsigned)(n_seqs * H), EG_THREADS, 0, stream>>>(
+                log_a, b, floor_, state, row_floats, m_off, (const bf16_t*)proj, p_ld, i_off, f_off, bias_i, bias_f, cap, cu_tokens,
+                state_slots, H);
+        IA_LAUNCH_CHECK("exp_gates (blocks)");
+        return 0;
+    }
     const unsigned blocks = (unsigned)((n_seqs * H + 63) / 64);
     if (dtype == IA_F32)
         exp_gates_kernel<float><<<blocks, 64, 0, stream>>>(log_a, b, floor_, state, row_floats, m_off, (const float*)proj, p_ld,
@@ -172,13 +238,22 @@ extern "C" int ia_step_gates(float* log_a, float* b, const void* proj, long long
     return 0;
 }
 
-// ---- the recurrence, token by token -----------------------------------------------------------------------------------
-// A block owns a (request, head, tile of S's columns) and walks the request's tokens in order.  A column j of S is
-// shared by P neighbouring lanes, each with LS_R of the column's `dim` entries in registers; the lanes add up q . S[:, j]
-// by a butterfly.  The next token's operands are asked for while this one is computed.  Nothing in the order of the sums
-// depends on how the tokens were cut into steps or on the batch.
+// ---- the recurrence ---------------------------------------------------------------------------------------------------
+// A block owns a (request, head, tile of S's columns) and walks tokens in order.  A column j of S is shared by P
+// neighbouring lanes, each with LS_R of the column's `dim` entries in registers; the lanes add up q . S[:, j] by a
+// butterfly.  The operands of a stage of tokens (q, k, the block's columns of v, decays, input scales) come into shared
+// memory together, already scaled, and the walk over the stage reads them from there.
+//
+// Three forms of one loop.  WALK: the request's tokens of this step from its state row and back into it (decode steps,
+// short portions).  Long portions are cut into chunks of `chunk` tokens that run side by side: LOCAL walks a chunk from
+// a state of zero, writes the chunk's outputs as if nothing came before it and leaves the chunk's final matrix and the
+// product of its decays in a workspace; `chunk_states_kernel` then walks a request's chunks in order, S <- A_c S + U_c
+// from the state row, leaving in the workspace the matrix each chunk starts from and in the state row the last one;
+// CARRY adds to every output of a chunk what the matrix it started from contributes, (prod_(s<=t) a_s) S_c^T q_t.
+// A token's result differs between the forms, and between chunk borders, by rounding only.
 #define LS_R 8
 #define LS_THREADS 256
+enum { LS_WALK = 0, LS_LOCAL = 1, LS_CARRY = 2 };
 
 struct ScanArgs {
     float* out;                 // [n][H][vdim]
@@ -193,74 +268,145 @@ struct ScanArgs {
     const int* cu_tokens; const int* state_slots;
     int H, dim, vdim, P, cols;                                    // cols: columns of S a block (LS_THREADS / P)
     float q_scale, k_scale;
+    int stage;                                                    // tokens whose operands a block holds in shared memory at a time
+    int chunk, max_chunks;                                        // LOCAL, CARRY: tokens of a chunk; chunks of the longest portion
+    float* chunk_s;                                               // [seqs][max_chunks][H][vt][dim]
+    float* chunk_a;                                               // [seqs][max_chunks][H]
 };
 
-template <typename T>
+template <typename T, int MODE, int P>
 __global__ __launch_bounds__(LS_THREADS) void linear_scan_kernel(const ScanArgs a) {
-    const int P = a.P;
+    // a stage of tokens: q and k [stage][P * LS_R] (scaled, zeros beyond dim), the block's columns of v [stage][cols],
+    // the decays and input scales [stage]
+    extern __shared__ __attribute__((aligned(16))) float ls_stage[];
+    constexpr int dimp = P * LS_R;                                // (P is a constant so that the butterfly runs on lane swaps)
+    float* const q_s = ls_stage;
+    float* const k_s = q_s + (size_t)a.stage * dimp;
+    float* const v_s = k_s + (size_t)a.stage * dimp;
+    float* const a_s = v_s + (size_t)a.stage * a.cols;
+    float* const b_s = a_s + a.stage;
     const int p = threadIdx.x % P, jj = threadIdx.x / P;
-    const int h = blockIdx.y, seq = blockIdx.z;
+    const int h = blockIdx.y;
+    const int seq = MODE == LS_WALK ? blockIdx.z : blockIdx.z / a.max_chunks;
+    const int c = MODE == LS_WALK ? 0 : blockIdx.z - seq * a.max_chunks;
     const int vt = a.vdim + (a.den != nullptr ? 1 : 0);           // columns of S
-    const int j = blockIdx.x * a.cols + jj;
+    const int j0 = blockIdx.x * a.cols, j = j0 + jj;
     const bool live = j < vt;
     const bool ones = j >= a.vdim;                                // the column whose value is always 1
-    const int first = a.cu_tokens[seq], last = a.cu_tokens[seq + 1];
+    int first = a.cu_tokens[seq], last = a.cu_tokens[seq + 1];
+    if (MODE != LS_WALK) {
+        first += c * a.chunk;
+        if (first >= last) return;                                // (the whole block: this request has fewer chunks)
+        last = first + a.chunk < last ? first + a.chunk : last;
+    }
     const int qh = h / (a.H / a.q_heads), kh = h / (a.H / a.k_heads);
     const int i0 = p * LS_R;
-    const T* q = (const T*)a.q + a.q_off + (long long)qh * a.dim + i0;
-    const T* k = (const T*)a.k + a.k_off + (long long)kh * a.dim + i0;
-    const T* v = (const T*)a.v + a.v_off + (long long)h * a.vdim + (ones || !live ? 0 : j);
-    float* srow = a.state + (long long)a.state_slots[seq] * a.row_floats + a.s_off +
-                  ((long long)h * vt + (live ? j : 0)) * a.dim + i0;
+    const T* q = (const T*)a.q + a.q_off + (long long)qh * a.dim;
+    const T* k = (const T*)a.k + a.k_off + (long long)kh * a.dim;
+    const T* v = (const T*)a.v + a.v_off + (long long)h * a.vdim;
+    const long long col = ((long long)h * vt + (live ? j : 0)) * a.dim + i0;
+    float* srow = MODE == LS_WALK ? a.state + (long long)a.state_slots[seq] * a.row_floats + a.s_off + col
+                                  : a.chunk_s + (long long)blockIdx.z * a.H * vt * a.dim + col;
     float S[LS_R];
 #pragma unroll
-    for (int r = 0; r < LS_R; ++r) S[r] = (live && i0 + r < a.dim) ? srow[r] : 0.f;
+    for (int r = 0; r < LS_R; ++r) S[r] = (MODE != LS_LOCAL && live && i0 + r < a.dim) ? srow[r] : 0.f;
     const float skip = a.skip != nullptr ? a.skip[h] : 0.f;
-
-    float qn[LS_R], kn[LS_R], vn = 0.f, an = 0.f, bn = 1.f;
-    auto fetch = [&](int t) {
-#pragma unroll
-        for (int r = 0; r < LS_R; ++r) {
-            const bool in = i0 + r < a.dim;
-            qn[r] = in ? ld(q + (long long)t * a.q_ld + r) : 0.f;
-            kn[r] = in ? ld(k + (long long)t * a.k_ld + r) : 0.f;
+    float run = 1.f;                                              // the product of the decays so far
+    for (int t0 = first; t0 < last; t0 += a.stage) {
+        const int nt = last - t0 < a.stage ? last - t0 : a.stage;
+        __syncthreads();                                          // (the stage before is used up)
+        for (int e = threadIdx.x; e < nt * dimp; e += LS_THREADS) {
+            const int tt = e / dimp, i = e - tt * dimp;
+            q_s[e] = i < a.dim ? ld(q + (long long)(t0 + tt) * a.q_ld + i) * a.q_scale : 0.f;
+            if (MODE != LS_CARRY) k_s[e] = i < a.dim ? ld(k + (long long)(t0 + tt) * a.k_ld + i) * a.k_scale : 0.f;
         }
-        vn = ones ? 1.f : ld(v + (long long)t * a.v_ld);
-        an = a.log_a[a.a_per_token ? (long long)t * a.H + h : h];
-        bn = a.b != nullptr ? a.b[(long long)t * a.H + h] : 1.f;
-    };
-    if (first < last) fetch(first);
-    for (int t = first; t < last; ++t) {
-        float qc[LS_R], kc[LS_R];
-#pragma unroll
-        for (int r = 0; r < LS_R; ++r) { qc[r] = qn[r] * a.q_scale; kc[r] = kn[r] * a.k_scale; }
-        const float vc = vn, decay = a.a_per_token ? expf(an) : an, bv = bn * vn;
-        if (t + 1 < last) fetch(t + 1);
-        float part = 0.f;
-#pragma unroll
-        for (int r = 0; r < LS_R; ++r) {
-            S[r] = fmaf(decay, S[r], bv * kc[r]);
-            part = fmaf(S[r], qc[r], part);
+        if (MODE != LS_CARRY)
+            for (int e = threadIdx.x; e < nt * a.cols; e += LS_THREADS) {
+                const int tt = e / a.cols, jv = j0 + e - tt * a.cols;
+                v_s[e] = jv < a.vdim ? ld(v + (long long)(t0 + tt) * a.v_ld + jv) : 1.f;
+            }
+        for (int e = threadIdx.x; e < nt; e += LS_THREADS) {
+            const float an = a.log_a[a.a_per_token ? (long long)(t0 + e) * a.H + h : h];
+            a_s[e] = a.a_per_token ? expf(an) : an;
+            b_s[e] = a.b != nullptr ? a.b[(long long)(t0 + e) * a.H + h] : 1.f;
         }
-        for (int o = P / 2; o > 0; o >>= 1) part += __shfl_xor(part, o, IA_WAVE);
-        if (p == 0 && live) {
-            if (ones) a.den[(long long)t * a.H + h] = part;
-            else a.out[((long long)t * a.H + h) * a.vdim + j] = fmaf(skip, vc, part);
+        __syncthreads();
+#pragma unroll 2
+        for (int tt = 0; tt < nt; ++tt) {
+            const float4 qa = *(const float4*)(q_s + tt * dimp + i0), qb = *(const float4*)(q_s + tt * dimp + i0 + 4);
+            const float qc[LS_R] = {qa.x, qa.y, qa.z, qa.w, qb.x, qb.y, qb.z, qb.w};
+            const float decay = a_s[tt];
+            run *= decay;
+            float part = 0.f, vc = 0.f;
+            if (MODE != LS_CARRY) {
+                const float4 ka = *(const float4*)(k_s + tt * dimp + i0), kb = *(const float4*)(k_s + tt * dimp + i0 + 4);
+                const float kc[LS_R] = {ka.x, ka.y, ka.z, ka.w, kb.x, kb.y, kb.z, kb.w};
+                vc = v_s[tt * a.cols + jj];
+                const float bv = b_s[tt] * vc;
+#pragma unroll
+                for (int r = 0; r < LS_R; ++r) S[r] = fmaf(decay, S[r], bv * kc[r]);
+            }
+#pragma unroll
+            for (int r = 0; r < LS_R; ++r) part = fmaf(S[r], qc[r], part);
+#pragma unroll
+            for (int o = P / 2; o > 0; o >>= 1) part += __shfl_xor(part, o, IA_WAVE);
+            if (p == 0 && live) {
+                const int t = t0 + tt;
+                float* at = ones ? a.den + (long long)t * a.H + h : a.out + ((long long)t * a.H + h) * a.vdim + j;
+                if (MODE == LS_CARRY) *at = fmaf(run, part, *at);
+                else *at = ones ? part : fmaf(skip, vc, part);
+            }
         }
     }
+    if (MODE == LS_CARRY) return;
     if (live)
 #pragma unroll
         for (int r = 0; r < LS_R; ++r)
             if (i0 + r < a.dim) srow[r] = S[r];
+    if (MODE == LS_LOCAL && blockIdx.x == 0 && threadIdx.x == 0) a.chunk_a[(long long)blockIdx.z * a.H + h] = run;
 }
 
+// A request's chunks in order, one thread an entry of the heads' matrices: the workspace's U_c becomes the matrix that
+// chunk c starts from, the state row takes the matrix behind the last chunk.
+__global__ void chunk_states_kernel(float* __restrict__ chunk_s, const float* __restrict__ chunk_a, float* __restrict__ state,
+                                    long long row_floats, long long s_off, const int* __restrict__ cu_tokens,
+                                    const int* __restrict__ state_slots, int per_head, int H, int chunk, int max_chunks) {
+    const long long e = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    const long long per_seq = (long long)H * per_head;
+    if (e >= per_seq) return;
+    const int seq = blockIdx.y;
+    const int h = (int)(e / per_head);
+    const int n_tokens = cu_tokens[seq + 1] - cu_tokens[seq];
+    const int chunks = (n_tokens + chunk - 1) / chunk;
+    float* srow = state + (long long)state_slots[seq] * row_floats + s_off + e;
+    float S = *srow;
+    for (int c = 0; c < chunks; ++c) {
+        const long long unit = (long long)seq * max_chunks + c;
+        float* u = chunk_s + unit * per_seq + e;
+        const float mine = *u;
+        *u = S;
+        S = fmaf(chunk_a[unit * H + h], S, mine);
+    }
+    *srow = S;
+}
+
+extern "C" long long ia_linear_scan_workspace(int n_seqs, int max_q_len, int chunk, int H, int dim, int vdim, int normaliser) {
+    if (chunk <= 0 || n_seqs <= 0) return 0;
+    const long long max_chunks = (max_q_len + chunk - 1) / chunk;
+    return (long long)n_seqs * max_chunks * ((long long)H * (vdim + (normaliser ? 1 : 0)) * dim + H);
+}
+
+// chunk 0: every request's tokens are walked from its state row.  chunk > 0: portions are cut into chunks of that many
+// tokens that run side by side; `workspace` holds ia_linear_scan_workspace(...) floats and max_q_len is an upper bound
+// of the tokens a request brings.
 extern "C" int ia_linear_scan(float* out, float* den, float* state, long long row_floats, long long s_off,
                               const void* q, long long q_ld, int q_off, int q_heads,
                               const void* k, long long k_ld, int k_off, int k_heads,
                               const void* v, long long v_ld, int v_off,
                               const float* log_a, int a_per_token, const float* b, const float* skip,
                               const int* cu_tokens, const int* state_slots, int n_seqs, int H, int dim, int vdim,
-                              float q_scale, float k_scale, int dtype, hipStream_t stream) {
+                              float q_scale, float k_scale, int chunk, int max_q_len, float* workspace, int dtype,
+                              hipStream_t stream) {
     IA_CHECK(n_seqs >= 0 && H > 0 && dim > 0 && vdim > 0, "linear_scan: bad sizes heads=%d dim=%d vdim=%d", H, dim, vdim);
     IA_CHECK(dim <= LS_R * IA_WAVE, "linear_scan: a key size of %d is beyond %d", dim, LS_R * IA_WAVE);
     IA_CHECK(q_heads > 0 && k_heads > 0 && H % q_heads == 0 && H % k_heads == 0,
@@ -269,6 +415,8 @@ extern "C" int ia_linear_scan(float* out, float* den, float* state, long long ro
     IA_CHECK(s_off >= 0 && s_off + (long long)H * vt * dim <= row_floats, "linear_scan: the matrices do not fit the state row");
     IA_CHECK(q_off >= 0 && q_off + (long long)q_heads * dim <= q_ld && k_off >= 0 && k_off + (long long)k_heads * dim <= k_ld &&
              v_off >= 0 && v_off + (long long)H * vdim <= v_ld, "linear_scan: q, k or v lie outside their rows");
+    IA_CHECK(chunk >= 0 && (chunk == 0 || (workspace != nullptr && max_q_len >= 1)), "linear_scan: chunks of %d tokens need a "
+             "workspace and the longest portion's length", chunk);
     if (n_seqs == 0) return 0;
     int P = 1;
     while (P * LS_R < dim) P *= 2;
@@ -281,10 +429,51 @@ extern "C" int ia_linear_scan(float* out, float* den, float* state, long long ro
     a.cu_tokens = cu_tokens; a.state_slots = state_slots;
     a.H = H; a.dim = dim; a.vdim = vdim; a.P = P; a.cols = LS_THREADS / P;
     a.q_scale = q_scale; a.k_scale = k_scale;
-    const dim3 grid((unsigned)((vt + a.cols - 1) / a.cols), (unsigned)H, (unsigned)n_seqs);
-    if (dtype == IA_F32) linear_scan_kernel<float><<<grid, LS_THREADS, 0, stream>>>(a);
-    else linear_scan_kernel<bf16_t><<<grid, LS_THREADS, 0, stream>>>(a);
-    IA_LAUNCH_CHECK("linear_scan");
+    a.chunk = chunk; a.max_chunks = chunk ? (max_q_len + chunk - 1) / chunk : 1;
+    a.chunk_s = workspace;
+    a.chunk_a = workspace ? workspace + (long long)n_seqs * a.max_chunks * H * vt * dim : nullptr;
+    IA_CHECK((long long)n_seqs * a.max_chunks <= 65535, "linear_scan: %d requests x %d chunks exceed the grid", n_seqs, a.max_chunks);
+    const unsigned tiles = (unsigned)((vt + a.cols - 1) / a.cols);
+    // a stage: as many tokens as 32 KB of shared memory hold (2 to 32), no more than a walk can have
+    const int per_token = 2 * P * LS_R + a.cols + 2;
+    int stage = 32 * 1024 / 4 / per_token;
+    stage = stage > 32 ? 32 : stage < 2 ? 2 : stage;
+    const int longest = chunk ? chunk : (max_q_len >= 1 ? max_q_len : 1);
+    a.stage = stage < longest ? stage : longest;
+    const size_t shm = (size_t)a.stage * per_token * sizeof(float);
+#define LS_LAUNCH_P(MODE, GRID, PP)                                                                            \
+    do {                                                                                                       \
+        if (dtype == IA_F32) linear_scan_kernel<float, MODE, PP><<<GRID, LS_THREADS, shm, stream>>>(a);        \
+        else linear_scan_kernel<bf16_t, MODE, PP><<<GRID, LS_THREADS, shm, stream>>>(a);                       \
+    } while (0)
+#define LS_LAUNCH(MODE, GRID)                                                                                  \
+    do {                                                                                                       \
+        switch (P) {                                                                                           \
+            case 1: LS_LAUNCH_P(MODE, GRID, 1); break;                                                         \
+            case 2: LS_LAUNCH_P(MODE, GRID, 2); break;                                                         \
+            case 4: LS_LAUNCH_P(MODE, GRID, 4); break;                                                         \
+            case 8: LS_LAUNCH_P(MODE, GRID, 8); break;                                                         \
+            case 16: LS_LAUNCH_P(MODE, GRID, 16); break;                                                       \
+            case 32: LS_LAUNCH_P(MODE, GRID, 32); break;                                                       \
+            default: LS_LAUNCH_P(MODE, GRID, 64); break;                                                       \
+        }                                                                                                      \
+    } while (0)
+    if (chunk == 0) {
+        const dim3 grid(tiles, (unsigned)H, (unsigned)n_seqs);
+        LS_LAUNCH(LS_WALK, grid);
+        IA_LAUNCH_CHECK("linear_scan");
+        return 0;
+    }
+    const dim3 grid(tiles, (unsigned)H, (unsigned)(n_seqs * a.max_chunks));
+    const int per_head = vt * dim;
+    const dim3 sgrid((unsigned)(((long long)H * per_head + 255) / 256), (unsigned)n_seqs);
+    LS_LAUNCH(LS_LOCAL, grid);
+    chunk_states_kernel<<<sgrid, 256, 0, stream>>>(a.chunk_s, a.chunk_a, state, row_floats, s_off, cu_tokens, state_slots, per_head,
+                                                   H, chunk, a.max_chunks);
+    LS_LAUNCH(LS_CARRY, grid);
+#undef LS_LAUNCH
+#undef LS_LAUNCH_P
+    IA_LAUNCH_CHECK("linear_scan (chunks)");
     return 0;
 }
 
@@ -334,6 +523,40 @@ __global__ __launch_bounds__(256) void group_norm_gate_kernel(
     }
 }
 
+// The same with a block a (token, group), for groups of many features.
+template <typename T>
+__global__ __launch_bounds__(256) void group_norm_gate_block_kernel(
+    T* __restrict__ out, const float* __restrict__ o, const float* __restrict__ den, const float* __restrict__ floor_,
+    int head, const T* __restrict__ gate, long long g_ld, int g_off, int act, int gate_first,
+    const float* __restrict__ w, float eps, int inner, int group) {
+    __shared__ float scratch[16];
+    const int per_row = inner / group;
+    const long long t = blockIdx.x / per_row;
+    const int c0 = (int)(blockIdx.x - t * per_row) * group;
+    const int H = inner / head;
+    auto value = [&](int c) {
+        float y = o[t * inner + c];
+        if (den != nullptr) {
+            const long long at = t * H + c / head;
+            y = y / (fmaxf(fabsf(den[at]), floor_[at]) + 1e-6f);
+        }
+        if (gate != nullptr && gate_first) y *= ls_gate(ld(gate + t * g_ld + g_off + c), act);
+        return y;
+    };
+    float sq = 0.f;
+    for (int c = c0 + threadIdx.x; c < c0 + group; c += blockDim.x) {
+        const float y = value(c);
+        sq = fmaf(y, y, sq);
+    }
+    const float rs = 1.0f / sqrtf(block_sum(sq, scratch) / (float)group + eps);
+    for (int c = c0 + threadIdx.x; c < c0 + group; c += blockDim.x) {
+        float y = value(c) * rs;
+        if (w != nullptr) y *= w[c];
+        if (gate != nullptr && !gate_first) y *= ls_gate(ld(gate + t * g_ld + g_off + c), act);
+        st(out + t * inner + c, y);
+    }
+}
+
 extern "C" int ia_group_norm_gate(void* out, const float* o, const float* den, const float* floor_, int head,
                                   const void* gate, long long g_ld, int g_off, int act, int gate_first, const float* w,
                                   float eps, int n, int inner, int group, int dtype, hipStream_t stream) {
@@ -344,6 +567,18 @@ extern "C" int ia_group_norm_gate(void* out, const float* o, const float* den, c
              "group_norm_gate: gate activation %d (1 SiLU, 4 sigmoid) at %d of %lld", act, g_off, g_ld);
     if (n == 0) return 0;
     const long long units = (long long)n * (inner / group);
+    IA_CHECK(units < 2147483647LL, "group_norm_gate: %d tokens x %d groups exceed the grid", n, inner / group);
+    if (group > 256) {
+        if (dtype == IA_F32)
+            group_norm_gate_block_kernel<float><<<(unsigned)units, 256, 0, stream>>>((float*)out, o, den, floor_, head, (const float*)gate,
+                                                                                  g_ld, g_off, act, gate_first, w, eps, inner, group);
+        else
+            group_norm_gate_block_kernel<bf16_t><<<(unsigned)units, 256, 0, stream>>>((bf16_t*)out, o, den, floor_, head,
+                                                                                   (const bf16_t*)gate, g_ld, g_off, act, gate_first, w,
+                                                                                   eps, inner, group);
+        IA_LAUNCH_CHECK("group_norm_gate (blocks)");
+        return 0;
+    }
     const unsigned blocks = (unsigned)((units + 3) / 4);
     if (dtype == IA_F32)
         group_norm_gate_kernel<float><<<blocks, 256, 0, stream>>>((float*)out, o, den, floor_, head, (const float*)gate, g_ld, g_off,

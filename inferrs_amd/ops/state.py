@@ -15,6 +15,9 @@ from . import KernelError, _DT, _check, _dev, _dt, _f32, _i32, _p, _stream, libr
 
 ACT_SILU, ACT_GELU_TANH, ACT_GELU, ACT_SIGMOID = 1, 2, 3, 4
 SCAN_MAX_DIM = 512            # rows of a head's matrix that the recurrence kernel takes
+SCAN_CHUNK = 64               # tokens of a chunk when long portions run in chunks side by side
+SCAN_CHUNKS_FROM = 128        # steps whose longest portion has more tokens than this run in chunks
+SCAN_WORKSPACE_FLOATS = 1 << 28   # the chunks' matrices take no more than this (1 GiB): longer chunks beyond
 
 
 # ---- the stream ---------------------------------------------------------------------------------------------------
@@ -96,11 +99,13 @@ def conv_act_step(x: torch.Tensor, x_off: int, channels: int, taps: torch.Tensor
 
 
 def exp_gates(proj: torch.Tensor, i_off: int, f_off: int, bias_i: torch.Tensor, bias_f: torch.Tensor, cap: float,
-              state: torch.Tensor, m_off: int, cu_tokens: torch.Tensor, state_slots: torch.Tensor
+              state: torch.Tensor, m_off: int, cu_tokens: torch.Tensor, state_slots: torch.Tensor, max_q_len: int = 0
               ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """Exponential gates under a running maximum: with i = cap tanh((proj_i + bias_i) / cap), f = logsigmoid(cap
     tanh((proj_f + bias_f) / cap)) and m_t = max(f + m_(t-1), i) (kept at `m_off` of the state row), returns 32-bit
-    (log decay f + m_(t-1) - m_t, input scale exp(i - m_t), floor exp(-m_t)), each [n, heads]."""
+    (log decay f + m_(t-1) - m_t, input scale exp(i - m_t), floor exp(-m_t)), each [n, heads].  `max_q_len`: an upper
+    bound of the tokens a request brings (0: unknown, the step's tokens); long portions are walked by a block's threads side
+    by side, which differs from the walk token by token by rounding."""
     _dev(proj, bias_i, bias_f, state, cu_tokens, state_slots)
     _f32(bias_i, "bias_i"); _f32(bias_f, "bias_f"); _i32(cu_tokens, "cu_tokens"); _i32(state_slots, "state_slots")
     row = _state(state)
@@ -110,7 +115,7 @@ def exp_gates(proj: torch.Tensor, i_off: int, f_off: int, bias_i: torch.Tensor, 
     outs = [torch.empty((n, H), dtype=torch.float32, device=proj.device) for _ in range(3)]
     _check(library().ia_exp_gates(_p(outs[0]), _p(outs[1]), _p(outs[2]), _p(state), row, m_off, _p(proj), proj.shape[1],
                                   i_off, f_off, _p(bias_i), _p(bias_f), ctypes.c_float(cap), _p(cu_tokens), _p(state_slots),
-                                  H, state_slots.numel(), _dt(proj), _stream()))
+                                  H, state_slots.numel(), int(max_q_len) or n, _dt(proj), _stream()))
     return outs[0], outs[1], outs[2]
 
 
@@ -133,12 +138,16 @@ def linear_scan(*, q: torch.Tensor, q_off: int, q_heads: int, k: torch.Tensor, k
                 cu_tokens: torch.Tensor, state_slots: torch.Tensor, log_a: Optional[torch.Tensor] = None,
                 decay: Optional[torch.Tensor] = None, b: Optional[torch.Tensor] = None,
                 skip: Optional[torch.Tensor] = None, q_scale: float = 1.0, k_scale: float = 1.0,
-                normaliser: bool = False):
+                normaliser: bool = False, max_q_len: int = 0, chunk: Optional[int] = None):
     """The recurrence S <- a S + b k v^T, o = S^T q (+ skip v) over each request's tokens, from and into the
     [heads, vdim (+ 1), dim] floats at `s_off` of its state row.  q, k, v are 2-D rows of one precision; head h reads
     q[:, q_off + (h // (heads / q_heads)) * dim ...], likewise k, and v[:, v_off + h * vdim ...].  The decay is `log_a`
     [n, heads] (logarithms, a (token, head)) or `decay` [heads] (constants); `b` [n, heads] or 1.  `normaliser`: S has
-    one more column whose value is always 1; returns (o, that column's output [n, heads]).  o is 32-bit [n, heads * vdim]."""
+    one more column whose value is always 1; returns (o, that column's output [n, heads]).  o is 32-bit [n, heads * vdim].
+    `max_q_len`: an upper bound of the tokens a request brings (0: unknown, the step's tokens).  `chunk`: 0 walks every
+    request's tokens in order; a number cuts portions into chunks of that many tokens that run side by side (three
+    kernels: each chunk from nothing, the chunks' matrices in order, what each chunk's start contributes), which differs
+    from the walk by rounding; None: chunks of `SCAN_CHUNK` for steps with a portion of more than `SCAN_CHUNKS_FROM` tokens."""
     _dev(q, k, v, state, cu_tokens, state_slots, log_a, decay, b, skip)
     _f32(log_a, "log_a"); _f32(decay, "decay"); _f32(b, "b"); _f32(skip, "skip")
     _i32(cu_tokens, "cu_tokens"); _i32(state_slots, "state_slots")
@@ -157,10 +166,21 @@ def linear_scan(*, q: torch.Tensor, q_off: int, q_heads: int, k: torch.Tensor, k
     out = torch.empty((n, heads * vdim), dtype=torch.float32, device=q.device)
     den = torch.empty((n, heads), dtype=torch.float32, device=q.device) if normaliser else None
     a = log_a if log_a is not None else decay
-    _check(library().ia_linear_scan(
+    n_seqs = state_slots.numel()
+    longest = int(max_q_len) or n
+    if chunk is None:
+        chunk = SCAN_CHUNK if longest > SCAN_CHUNKS_FROM else 0
+        while chunk and n_seqs * -(-longest // chunk) * heads * (vdim + 1) * dim > SCAN_WORKSPACE_FLOATS:
+            chunk *= 2
+    lib = library()
+    work = None
+    if chunk:
+        work = torch.empty((lib.ia_linear_scan_workspace(n_seqs, longest, chunk, heads, dim, vdim, int(normaliser)),),
+                           dtype=torch.float32, device=q.device)
+    _check(lib.ia_linear_scan(
         _p(out), _p(den), _p(state), row, s_off, _p(q), q.shape[1], q_off, q_heads, _p(k), k.shape[1], k_off, k_heads,
         _p(v), v.shape[1], v_off, _p(a), int(log_a is not None), _p(b), _p(skip), _p(cu_tokens), _p(state_slots),
-        state_slots.numel(), heads, dim, vdim, ctypes.c_float(q_scale), ctypes.c_float(k_scale), _dt(q), _stream()))
+        n_seqs, heads, dim, vdim, ctypes.c_float(q_scale), ctypes.c_float(k_scale), chunk, longest, _p(work), _dt(q), _stream()))
     return (out, den) if normaliser else out
 
 

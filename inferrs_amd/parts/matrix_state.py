@@ -65,7 +65,7 @@ class Retention(Mixer):
         proj = self.proj(h)                                   # [n, q | k | v | g]
         o = ops.linear_scan(q=proj, q_off=0, q_heads=s.n_heads, k=proj, k_off=qk, k_heads=s.n_heads, v=proj, v_off=2 * qk,
                             heads=s.n_heads, dim=s.head_dim, vdim=s.v_dim, state=cache.state, s_off=0,
-                            cu_tokens=ctx.cu_tokens, state_slots=ctx.state_slots, decay=self.decay,
+                            cu_tokens=ctx.cu_tokens, state_slots=ctx.state_slots, decay=self.decay, max_q_len=ctx.max_q_len,
                             k_scale=s.head_dim ** -0.5)
         y = ops.group_norm_gate(o, group=s.v_dim, head=s.v_dim, eps=s.norm_eps, out_dtype=proj.dtype, gate=proj,
                                 gate_off=2 * qk + vv, act=ops.state.ACT_SILU)
@@ -105,10 +105,11 @@ class MatrixMemory(Mixer):
         proj = self.proj(h)                                   # [n, q | k | v | g | i | f]
         m_off = H * (s.v_dim + 1) * s.head_dim
         log_a, b, floor = ops.exp_gates(proj, 2 * qk + 2 * vv, 2 * qk + 2 * vv + H, self.bias_i, self.bias_f, s.gate_cap,
-                                        cache.state, m_off, ctx.cu_tokens, ctx.state_slots)
+                                        cache.state, m_off, ctx.cu_tokens, ctx.state_slots, max_q_len=ctx.max_q_len)
         o, den = ops.linear_scan(q=proj, q_off=0, q_heads=H, k=proj, k_off=qk, k_heads=H, v=proj, v_off=2 * qk, heads=H,
                                  dim=s.head_dim, vdim=s.v_dim, state=cache.state, s_off=0, cu_tokens=ctx.cu_tokens,
-                                 state_slots=ctx.state_slots, log_a=log_a, b=b, q_scale=s.head_dim ** -0.5, normaliser=True)
+                                 state_slots=ctx.state_slots, log_a=log_a, b=b, q_scale=s.head_dim ** -0.5, normaliser=True,
+                                 max_q_len=ctx.max_q_len)
         y = ops.group_norm_gate(o, group=s.v_dim, head=s.v_dim, eps=s.norm_eps, out_dtype=proj.dtype, weight=self.norm,
                                 gate=proj, gate_off=2 * qk + vv, act=ops.state.ACT_SIGMOID, den=den, floor=floor)
         return self.o(y)
@@ -160,7 +161,7 @@ class StateSpace(Mixer):
         log_a, b = ops.step_gates(proj, 2 * inner + 2 * bc, self.dt_bias, self.a_log)
         y = ops.linear_scan(q=xbc, q_off=inner + bc, q_heads=s.groups, k=xbc, k_off=inner, k_heads=s.groups, v=xbc, v_off=0,
                             heads=s.n_heads, dim=s.state, vdim=s.v_dim, state=cache.state, s_off=0, cu_tokens=ctx.cu_tokens,
-                            state_slots=ctx.state_slots, log_a=log_a, b=b, skip=self.skip)
+                            state_slots=ctx.state_slots, log_a=log_a, b=b, skip=self.skip, max_q_len=ctx.max_q_len)
         y = ops.group_norm_gate(y, group=inner // s.norm_groups, head=s.v_dim, eps=s.norm_eps, out_dtype=proj.dtype,
                                 weight=self.norm, gate=proj, gate_off=0, act=ops.state.ACT_SILU, gate_first=True)
         return self.o(y)

@@ -10,7 +10,9 @@ pool whose pages and state slots are used again), in both precisions, with ordin
 queries.  Decays are drawn so that some heads remember for hundreds of tokens: a state that is lost, not cleared or
 carried to the wrong request shows.  Greedy generation runs through the engine's own entry point and scheduler.
 
-Tolerances.  32-bit: 2e-5 of the largest logit against the 64-bit result, at every position.  bfloat16: the measure is
+Tolerances.  32-bit: 2e-5 of the largest logit against the 64-bit result, at every position; where the plain
+implementation's own 32-bit arithmetic is further off than a third of that (a head's output that nearly cancels in
+front of its norm), three times what it is off.  bfloat16: the measure is
 the distribution of the positions' errors against that of the plain implementation in bfloat16 arithmetic (every
 operation rounded) on the same positions: the engine keeps more in 32-bit than that, so its median and its ninth
 decile must not be larger (a tenth and a half of slack)."""
@@ -257,7 +259,8 @@ def test_matrix_state_carried_over_portions(kind):
         counts = [p.shape[0] for p in parts]
         ctx = SimpleNamespace(cu_tokens=dev(torch.tensor([0] + list(np.cumsum(counts)), dtype=torch.int32)),
                               token_seq=dev(torch.tensor([i for i, c in enumerate(counts) for _ in range(c)], dtype=torch.int32)),
-                              state_slots=dev(torch.tensor(live, dtype=torch.int32)), stream=None, partial_sums=False)
+                              state_slots=dev(torch.tensor(live, dtype=torch.int32)), stream=None, partial_sums=False,
+                              max_q_len=max(counts))
         out = part.forward(ctx, dev(torch.cat(parts)), LayerCache(0, state=state)).cpu()
         o = 0
         for s, c in zip(live, counts):
@@ -266,6 +269,65 @@ def test_matrix_state_carried_over_portions(kind):
     for s in lens:
         np.testing.assert_allclose(torch.cat(got[s]).numpy(), want[s].numpy(), rtol=3e-4, atol=3e-5)
     assert (state[[0, 2, 4]] == 7.0).all()                             # nobody else's row was touched
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("H,qh,dim,vdim,normaliser", [(3, 3, 10, 12, False), (4, 2, 24, 9, True), (2, 1, 128, 64, True), (8, 8, 64, 128, False)])
+def test_scan_in_chunks_is_the_walk(H, qh, dim, vdim, normaliser, dtype):
+    """Three requests of unequal lengths in one step, from states that are not zero: chunks of 16 and of 64 tokens side
+    by side give what the walk token by token gives, outputs and final states, up to rounding; so do decays that are
+    constants of the heads."""
+    from inferrs_amd import ops
+    g = torch.Generator().manual_seed(H * dim)
+    lens = [150, 1, 333]
+    n = sum(lens)
+    q = dev(torch.randn(n, qh * dim, generator=g), dtype)
+    k = dev(torch.randn(n, qh * dim, generator=g), dtype)
+    v = dev(torch.randn(n, H * vdim, generator=g), dtype)
+    log_a = dev(-torch.rand(n, H, generator=g) * torch.tensor([0.001, 0.05, 0.5, 3.0] * 2)[:H])
+    b = dev(torch.rand(n, H, generator=g))
+    decay = dev(torch.tensor([0.999, 0.5, 0.97, 1.0, 0.0, 0.9, 0.99, 0.8][:H]))
+    skip = dev(torch.randn(H, generator=g))
+    cu = dev(torch.tensor([0, 150, 151, 484], dtype=torch.int32))
+    slots = dev(torch.tensor([2, 0, 3], dtype=torch.int32))
+    floats = H * (vdim + int(normaliser)) * dim
+    start = torch.randn(5, floats + 7, generator=g)
+
+    def run(chunk, **gates):
+        state = dev(start.clone())
+        out = ops.linear_scan(q=q, q_off=0, q_heads=qh, k=k, k_off=0, k_heads=qh, v=v, v_off=0, heads=H, dim=dim, vdim=vdim,
+                              state=state, s_off=7, cu_tokens=cu, state_slots=slots, skip=skip, q_scale=0.7, k_scale=dim ** -0.5,
+                              normaliser=normaliser, max_q_len=333, chunk=chunk, **gates)
+        outs = out if normaliser else (out,)
+        return [o.cpu().double() for o in outs] + [state.cpu().double()]
+
+    for gates in (dict(log_a=log_a, b=b), dict(decay=decay)):
+        walk = run(0, **gates)
+        assert torch.equal(walk[-1][[1, 4]], start[[1, 4]].double()) and torch.equal(walk[-1][:, :7], start[:, :7].double())
+        for chunk in (16, 64, None):
+            for got, want in zip(run(chunk, **gates), walk):
+                scale = float(want.abs().max())
+                assert float((got - want).abs().max()) <= 2e-5 * scale, (chunk, float((got - want).abs().max()) / scale)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_gates_of_long_portions_are_the_walk(dtype):
+    from inferrs_amd import ops
+    g = torch.Generator().manual_seed(3)
+    H, lens = 3, [700, 1, 40]
+    n = sum(lens)
+    proj = dev(4.0 * torch.randn(n, 2 * H + 5, generator=g), dtype)
+    bi, bf = dev(torch.randn(H, generator=g)), dev(torch.tensor([1.0, 4.0, -2.0]))
+    cu = dev(torch.tensor([0, 700, 701, 741], dtype=torch.int32))
+    slots = dev(torch.tensor([1, 2, 0], dtype=torch.int32))
+    start = torch.randn(3, H + 2, generator=g)
+    results = []
+    for longest in (1, 700):            # 1: the walk a (request, head); 700: a block's threads side by side
+        state = dev(start.clone())
+        outs = ops.exp_gates(proj, 2, 2 + H, bi, bf, 7.0, state, 2, cu, slots, max_q_len=longest)
+        results.append([o.cpu().double() for o in outs] + [state.cpu().double()])
+    for got, want in zip(results[1], results[0]):
+        assert float((got - want).abs().max()) <= 2e-5 * max(float(want.abs().max()), 1.0)
 
 
 # ---- whole models under every cutting ---------------------------------------------------------------
@@ -278,12 +340,18 @@ def models(tmp_path_factory):
         folder = str(tmp_path_factory.mktemp(f"lofudra_{name}"))
         tensors = write_model(folder, cfg, seed=11, sharpen=sharpen)
         reqs = {f"r{i}": random_tokens(n, cfg["vocab"], 40 + i) for i, n in enumerate(LENGTHS)}
-        ref = {r: pl.forward(cfg, tensors, t).numpy().astype(np.float32) for r, t in reqs.items()}
+        ref64 = {r: pl.forward(cfg, tensors, t) for r, t in reqs.items()}
+        ref = {r: v.numpy().astype(np.float32) for r, v in ref64.items()}
+        scale = max(float(v.abs().max()) for v in ref64.values())
+        # what rounding alone does at every position: the plain implementation in 32-bit against itself in 64-bit
+        NOISE[(name, sharpen)] = {r: ((pl.forward(cfg, tensors, t, dtype=torch.float32).double() - ref64[r]).abs().max(1).values
+                                      / scale).numpy() for r, t in reqs.items()}
         out[(name, sharpen)] = (folder, cfg, tensors, reqs, ref)
     return out
 
 
 _ROUNDED = {}
+NOISE = {}
 
 
 def rounded_errors(key, models):
@@ -346,8 +414,10 @@ def test_every_cutting_matches_plain(models, tmp_path, case, dtype):
         got = replay(folder, cfg, dtype, trace, str(tmp_path / f"{mode}_{dtype}"), page=16 if mode != "mixed2" else 32)
         part = {r: reqs[r] for r in got}
         if dtype == "float32":
-            err, where = worst(got, ref, part)
-            assert err <= TOL_F32, f"{case} {dtype} {mode}: {err:.3g} of the scale at {where}, allowed {TOL_F32:.3g}"
+            for r, e in errors(got, ref, part).items():
+                allowed = np.maximum(TOL_F32, 3.0 * NOISE[case][r])
+                assert (e <= allowed).all(), (f"{case} {dtype} {mode}: {float(e[np.argmax(e / allowed)]):.3g} of the scale at "
+                                              f"({r}, {int(np.argmax(e / allowed))}), allowed {float(allowed[np.argmax(e / allowed)]):.3g}")
             continue
         plain = rounded_errors(case, models)
         common = [r for r in part if r in plain]
