@@ -41,6 +41,60 @@ __global__ void conv_act_kernel(T* __restrict__ out, const T* __restrict__ x, co
     st(out + i, acc);
 }
 
+// The same for bfloat16 rows, eight neighbouring channels a thread (16-byte accesses): channels, row length and
+// offset in steps of 8.  The sums are those of the kernel above.
+typedef uint32_t ls_u32x4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void ls_unpack8(const bf16_t* p, float (&v)[8]) {
+    const ls_u32x4 q = *reinterpret_cast<const ls_u32x4*>(p);
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+        v[2 * e] = __uint_as_float(q[e] << 16);
+        v[2 * e + 1] = __uint_as_float(q[e] & 0xffff0000u);
+    }
+}
+
+__global__ void conv_act8_kernel(bf16_t* __restrict__ out, const bf16_t* __restrict__ x, const bf16_t* __restrict__ taps,
+                                 const bf16_t* __restrict__ bias, const float* __restrict__ state, long long row_floats,
+                                 long long tail_off, const int* __restrict__ token_seq, const int* __restrict__ cu_tokens,
+                                 const int* __restrict__ state_slots, int C, int k, long long x_ld, int x_off, int act,
+                                 long long total8) {
+    const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total8) return;
+    const int per_row = C / 8;
+    const int t = (int)(i / per_row), c = (int)(i - (long long)t * per_row) * 8;
+    const int seq = token_seq[t];
+    const int first = cu_tokens[seq];
+    const float* tail = state + (long long)state_slots[seq] * row_floats + tail_off + c;
+    float acc[8];
+    if (bias != nullptr) ls_unpack8(bias + c, acc);
+    else {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = 0.f;
+    }
+    for (int j = 0; j < k; ++j) {
+        const int src = t - (k - 1 - j);
+        float v[8], tp[8];
+        ls_unpack8(taps + (long long)j * C + c, tp);
+        if (src >= first) {
+            ls_unpack8(x + (long long)src * x_ld + x_off + c, v);
+        } else {
+            const float* from = tail + (long long)((k - 1) + (src - first)) * C;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = from[e];
+        }
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = fmaf(tp[e], v[e], acc[e]);
+    }
+    if (act == IA_ACT_SILU) {
+#pragma unroll
+        for (int e = 0; e < 8; ++e) acc[e] = acc[e] / (1.0f + expf(-acc[e]));
+    }
+    ls_u32x4 q;
+    q[0] = pack_bf16x2(acc[0], acc[1]); q[1] = pack_bf16x2(acc[2], acc[3]);
+    q[2] = pack_bf16x2(acc[4], acc[5]); q[3] = pack_bf16x2(acc[6], acc[7]);
+    *reinterpret_cast<ls_u32x4*>(out + (long long)t * C + c) = q;
+}
+
 // After the convolution of a step: a request's tail takes the last k - 1 inputs, oldest first.
 template <typename T>
 __global__ void conv_tail_kernel(float* __restrict__ state, long long row_floats, long long tail_off,
@@ -81,6 +135,13 @@ extern "C" int ia_conv_act_step(void* out, const void* x, const void* taps, cons
             conv_tail_kernel<float><<<tail_grid, 256, 0, stream>>>(state, row_floats, tail_off, (const float*)x, cu_tokens,
                                                                    state_slots, C, k, x_ld, x_off);
     } else {
+        const bool wide = C % 8 == 0 && x_ld % 8 == 0 && x_off % 8 == 0 && tail_off % 4 == 0 && row_floats % 4 == 0 &&
+                          (((uintptr_t)out | (uintptr_t)x | (uintptr_t)taps | (uintptr_t)bias | (uintptr_t)state) & 15) == 0;
+        if (wide)
+            conv_act8_kernel<<<(unsigned)((total / 8 + 255) / 256), 256, 0, stream>>>(
+                (bf16_t*)out, (const bf16_t*)x, (const bf16_t*)taps, (const bf16_t*)bias, state, row_floats, tail_off, token_seq,
+                cu_tokens, state_slots, C, k, x_ld, x_off, act, total / 8);
+        else
         conv_act_kernel<bf16_t><<<blocks, 256, 0, stream>>>((bf16_t*)out, (const bf16_t*)x, (const bf16_t*)taps,
                                                             (const bf16_t*)bias, state, row_floats, tail_off, token_seq, cu_tokens,
                                                             state_slots, C, k, x_ld, x_off, act, total);
@@ -320,11 +381,13 @@ __global__ __launch_bounds__(LS_THREADS) void linear_scan_kernel(const ScanArgs 
             q_s[e] = i < a.dim ? ld(q + (long long)(t0 + tt) * a.q_ld + i) * a.q_scale : 0.f;
             if (MODE != LS_CARRY) k_s[e] = i < a.dim ? ld(k + (long long)(t0 + tt) * a.k_ld + i) * a.k_scale : 0.f;
         }
-        if (MODE != LS_CARRY)
-            for (int e = threadIdx.x; e < nt * a.cols; e += LS_THREADS) {
-                const int tt = e / a.cols, jv = j0 + e - tt * a.cols;
-                v_s[e] = jv < a.vdim ? ld(v + (long long)(t0 + tt) * a.v_ld + jv) : 1.f;
-            }
+        for (int e = threadIdx.x; e < nt * a.cols; e += LS_THREADS) {
+            const int tt = e / a.cols, jv = j0 + e - tt * a.cols;
+            if (MODE != LS_CARRY) v_s[e] = jv < a.vdim ? ld(v + (long long)(t0 + tt) * a.v_ld + jv) : 1.f;
+            // (CARRY: what the chunk's own walk left at the places this block adds to, so that no load stands in the walk)
+            else v_s[e] = jv < a.vdim ? a.out[((long long)(t0 + tt) * a.H + h) * a.vdim + jv]
+                                      : jv < vt ? a.den[(long long)(t0 + tt) * a.H + h] : 0.f;
+        }
         for (int e = threadIdx.x; e < nt; e += LS_THREADS) {
             const float an = a.log_a[a.a_per_token ? (long long)(t0 + e) * a.H + h : h];
             a_s[e] = a.a_per_token ? expf(an) : an;
@@ -353,7 +416,7 @@ __global__ __launch_bounds__(LS_THREADS) void linear_scan_kernel(const ScanArgs 
             if (p == 0 && live) {
                 const int t = t0 + tt;
                 float* at = ones ? a.den + (long long)t * a.H + h : a.out + ((long long)t * a.H + h) * a.vdim + j;
-                if (MODE == LS_CARRY) *at = fmaf(run, part, *at);
+                if (MODE == LS_CARRY) *at = fmaf(run, part, v_s[tt * a.cols + jj]);
                 else *at = ones ? part : fmaf(skip, vc, part);
             }
         }

@@ -272,6 +272,38 @@ def test_matrix_state_carried_over_portions(kind):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("C,ld,off,taps", [(64, 160, 32, 4), (56, 83, 24, 3), (128, 196, 64, 1), (8, 16, 8, 7)])
+def test_convolution_with_its_tail(C, ld, off, taps, dtype):
+    """Two requests fed in portions (shorter than the taps too) from slots 2 and 0 of a dirty state array: channel by
+    channel and, for bfloat16 rows whose sizes allow it, eight channels a thread."""
+    from inferrs_amd import ops
+    g = torch.Generator().manual_seed(C + taps)
+    lens = {2: 90, 0: 37}
+    x = {s: torch.randn(n, ld, generator=g).to(dtype) for s, n in lens.items()}
+    w, bias = (0.6 * torch.randn(C, taps, generator=g)).to(dtype), (0.2 * torch.randn(C, generator=g)).to(dtype)
+    want = {s: pl.silu(pl.causal_conv(x[s][:, off:off + C].double(), w.double(), bias.double())) for s in lens}
+    state = torch.full((3, 5 + (taps - 1) * C), 7.0, device="cuda")
+    state[2].zero_(); state[0].zero_()
+    cuts = {2: [1, 2, 1, 40, 3, 43], 0: [5, 1, 1, 30]}
+    at, got, step = {s: 0 for s in lens}, {s: [] for s in lens}, 0
+    while any(at[s] < lens[s] for s in lens):
+        live = [s for s in lens if at[s] < lens[s] and step < len(cuts[s])]
+        counts = [cuts[s][step] for s in live]
+        rows = dev(torch.cat([x[s][at[s]:at[s] + c] for s, c in zip(live, counts)]))
+        cu = dev(torch.tensor([0] + list(np.cumsum(counts)), dtype=torch.int32))
+        seq = dev(torch.tensor([i for i, c in enumerate(counts) for _ in range(c)], dtype=torch.int32))
+        out = ops.conv_act_step(rows, off, C, dev(w.t()), dev(bias), state, 5, seq, cu, dev(torch.tensor(live, dtype=torch.int32))).cpu()
+        o = 0
+        for s, c in zip(live, counts):
+            got[s].append(out[o:o + c]); o += c; at[s] += c
+        step += 1
+    for s in lens:
+        np.testing.assert_allclose(torch.cat(got[s]).double().numpy(), want[s].numpy(), rtol=1e-2 if dtype == torch.bfloat16 else 1e-5,
+                                   atol=1e-2 if dtype == torch.bfloat16 else 1e-5)
+    assert (state[1] == 7.0).all() and (state[:, :5].cpu() == torch.tensor([[0.0], [7.0], [0.0]])).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("H,qh,dim,vdim,normaliser", [(3, 3, 10, 12, False), (4, 2, 24, 9, True), (2, 1, 128, 64, True), (8, 8, 64, 128, False)])
 def test_scan_in_chunks_is_the_walk(H, qh, dim, vdim, normaliser, dtype):
     """Three requests of unequal lengths in one step, from states that are not zero: chunks of 16 and of 64 tokens side
