@@ -3,9 +3,9 @@
 config.json describes the model layer by layer:
 
     "architecture": "Lofudra", "vocab", "width", "norm": {"eps"},
-    "loop": {"start", "stop", "times"} (optional: layers start..stop-1 run `times` times in a row, each pass with a
-    cache or state of its own; before every pass row t of the tensor "loop.step" enters the stream, and before every
-    pass but the first the embedding's output once more),
+    "loop": {"start", "stop", "times"} (optional: the layers from `start` up to but not including `stop` are walked
+    `times` times over before the model goes on, every walk keeping caches and states of its own; row t of the tensor
+    "loop.step" enters the stream ahead of walk t, and ahead of every walk but the first so does the embedding's output),
     "layers": [{"type": "parallel" | "mlstm" | "mamba2", "mixer": {...}, "mlp": {"kind": "dense", "ff"} | null}, ...]
 
     mixer of "parallel": left: {heads, kv_heads, dim, vdim, scale, mask: {size}, rot: {base, dims}},

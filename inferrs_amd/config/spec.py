@@ -67,7 +67,7 @@ class AttentionSpec:
     qkv_bias: bool = False                 # q_proj.bias, k_proj.bias, v_proj.bias are added to the projections
     o_bias: bool = False                   # o_proj.bias is added to the output projection
     sink: bool = False                     # the softmax's denominator holds one more term, exp(0): a key of score 0 without a value
-    values_from_keys: bool = False         # no value projection: a value is its key as projected, before norm and rotation
+    values_from_keys: bool = False         # no value projection: a value is the key projection's own row, taken ahead of the per-head norm and the turn by position
     names: Optional[Tuple[Tuple[str, str], ...]] = None    # (the part's tensor name, the name in the file) where they differ
     kind: str = "attention"
 
@@ -98,9 +98,9 @@ class DenseMlpSpec:
 
 @dataclass(frozen=True)
 class RetentionSpec:
-    """Linear attention with a fixed decay a head and neither softmax nor denominator: k is scaled by dim^-1/2,
-    S <- decay_h S + k v^T, o = S^T q; each head's o is divided by its root mean square (`norm_eps`, no weight), the
-    joined heads are multiplied by silu(W_g h) and projected.  No biases."""
+    """A sum of outer products k v^T a head that fades by a constant factor a token and is read out with the query,
+    un-normalised: S <- decay_h S + (k dim^-1/2) v^T, o = S^T q.  A head's o then gets unit root mean square (`norm_eps`,
+    weightless); the heads side by side are gated by silu(W_g h) and go through W_o.  No biases anywhere."""
     hidden: int
     n_heads: int
     head_dim: int
@@ -128,8 +128,8 @@ class MatrixMemorySpec:
     """The matrix memory with exponential gates (the mLSTM of the xLSTM): q is scaled by dim^-1/2; a log input gate
     i = cap tanh((W_i h + b_i) / cap) and a log forget gate f = logsigmoid(cap tanh((W_f h + b_f) / cap)) a head; under a
     running maximum m_t = max(f + m_(t-1), i) that starts at 0, S <- exp(f + m_(t-1) - m_t) S + exp(i - m_t) k v^T and
-    n likewise with k alone; o = S^T q / (max(|n . q|, exp(-m_t)) + 1e-6); each head's o is divided by its root mean
-    square (`norm_eps`), the joined heads times a weight, times sigmoid(W_g h), projected."""
+    n likewise with k alone; o = S^T q / (max(|n . q|, exp(-m_t)) + 1e-6).  A head's o then gets unit root mean square
+    (`norm_eps`); the heads side by side are scaled by a weight vector, gated by sigmoid(W_g h) and go through W_o."""
     hidden: int
     n_heads: int
     head_dim: int
@@ -142,8 +142,8 @@ class MatrixMemorySpec:
 @dataclass(frozen=True)
 class StateSpaceSpec:
     """A selective state space with a scalar decay a head (Mamba-2): one product gives [z | x | B | C | dt] with
-    inner = n_heads * v_dim and `groups` groups of `state` entries for B and C; x, B and C pass a causal convolution a
-    channel (`conv` taps, a bias) and SiLU; dt = softplus(dt + dt_bias); S <- exp(-exp(A_log) dt) S + dt B x^T,
+    inner = n_heads * v_dim and `groups` groups of `state` entries for B and C; the channels of x, B and C are each
+    filtered over their last `conv` inputs (a bias, then SiLU); dt = softplus(dt + dt_bias); S <- exp(-exp(A_log) dt) S + dt B x^T,
     y = S^T C + D x; y * silu(z) is RMS-normed in `norm_groups` equal parts (`norm_eps`), times a weight, projected."""
     hidden: int
     n_heads: int

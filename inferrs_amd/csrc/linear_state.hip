@@ -329,6 +329,7 @@ struct ScanArgs {
     const int* cu_tokens; const int* state_slots;
     int H, dim, vdim, P, cols;                                    // cols: columns of S a block (LS_THREADS / P)
     float q_scale, k_scale;
+    int wide;                                                     // the matrices' rows start at multiples of 16 bytes
     int stage;                                                    // tokens whose operands a block holds in shared memory at a time
     int chunk, max_chunks;                                        // LOCAL, CARRY: tokens of a chunk; chunks of the longest portion
     float* chunk_s;                                               // [seqs][max_chunks][H][vt][dim]
@@ -368,9 +369,17 @@ __global__ __launch_bounds__(LS_THREADS) void linear_scan_kernel(const ScanArgs 
     const long long col = ((long long)h * vt + (live ? j : 0)) * a.dim + i0;
     float* srow = MODE == LS_WALK ? a.state + (long long)a.state_slots[seq] * a.row_floats + a.s_off + col
                                   : a.chunk_s + (long long)blockIdx.z * a.H * vt * a.dim + col;
+    // (a thread's eight entries as two 16-byte accesses where the matrices' rows allow it: a decode step is this read
+    // and the write at the end)
+    const bool wide = a.wide && i0 + LS_R <= a.dim;
     float S[LS_R];
+    if (MODE != LS_LOCAL && live && wide) {
+        const float4 lo = *(const float4*)srow, hi = *(const float4*)(srow + 4);
+        S[0] = lo.x; S[1] = lo.y; S[2] = lo.z; S[3] = lo.w; S[4] = hi.x; S[5] = hi.y; S[6] = hi.z; S[7] = hi.w;
+    } else {
 #pragma unroll
-    for (int r = 0; r < LS_R; ++r) S[r] = (MODE != LS_LOCAL && live && i0 + r < a.dim) ? srow[r] : 0.f;
+        for (int r = 0; r < LS_R; ++r) S[r] = (MODE != LS_LOCAL && live && i0 + r < a.dim) ? srow[r] : 0.f;
+    }
     const float skip = a.skip != nullptr ? a.skip[h] : 0.f;
     float run = 1.f;                                              // the product of the decays so far
     for (int t0 = first; t0 < last; t0 += a.stage) {
@@ -422,10 +431,14 @@ __global__ __launch_bounds__(LS_THREADS) void linear_scan_kernel(const ScanArgs 
         }
     }
     if (MODE == LS_CARRY) return;
-    if (live)
+    if (live && wide) {
+        *(float4*)srow = make_float4(S[0], S[1], S[2], S[3]);
+        *(float4*)(srow + 4) = make_float4(S[4], S[5], S[6], S[7]);
+    } else if (live) {
 #pragma unroll
         for (int r = 0; r < LS_R; ++r)
             if (i0 + r < a.dim) srow[r] = S[r];
+    }
     if (MODE == LS_LOCAL && blockIdx.x == 0 && threadIdx.x == 0) a.chunk_a[(long long)blockIdx.z * a.H + h] = run;
 }
 
@@ -494,6 +507,7 @@ extern "C" int ia_linear_scan(float* out, float* den, float* state, long long ro
     a.q_scale = q_scale; a.k_scale = k_scale;
     a.chunk = chunk; a.max_chunks = chunk ? (max_q_len + chunk - 1) / chunk : 1;
     a.chunk_s = workspace;
+    a.wide = dim % 4 == 0 && s_off % 4 == 0 && row_floats % 4 == 0 && ((uintptr_t)state & 15) == 0 && ((uintptr_t)workspace & 15) == 0;
     a.chunk_a = workspace ? workspace + (long long)n_seqs * a.max_chunks * H * vt * dim : nullptr;
     IA_CHECK((long long)n_seqs * a.max_chunks <= 65535, "linear_scan: %d requests x %d chunks exceed the grid", n_seqs, a.max_chunks);
     const unsigned tiles = (unsigned)((vt + a.cols - 1) / a.cols);
@@ -542,7 +556,7 @@ extern "C" int ia_linear_scan(float* out, float* den, float* state, long long ro
 
 // ---- what follows the recurrence: a norm a group of features, a gate, an optional division --------------------------
 //     y = o / (max(|den|, floor) + 1e-6)        (with den: the matrix memory's normaliser, a (token, head))
-//     y = y * act(g)                            (gate_first: the gate comes before the norm)
+//     y = y * act(g)                            (gate_first: gated, then normed)
 //     y = y / rms(y over its group) * w         (groups of `group` neighbouring features; w may be null)
 //     y = y * act(g)                            (otherwise the gate comes behind it)
 // One wave a (token, group); 32-bit throughout, rounded once when it is stored.  act: 1 SiLU, 4 sigmoid.
@@ -588,7 +602,7 @@ __global__ __launch_bounds__(256) void group_norm_gate_kernel(
 
 // The same with a block a (token, group), for groups of many features.
 template <typename T>
-__global__ __launch_bounds__(256) void group_norm_gate_block_kernel(
+__global__ __launch_bounds__(1024) void group_norm_gate_block_kernel(
     T* __restrict__ out, const float* __restrict__ o, const float* __restrict__ den, const float* __restrict__ floor_,
     int head, const T* __restrict__ gate, long long g_ld, int g_off, int act, int gate_first,
     const float* __restrict__ w, float eps, int inner, int group) {
@@ -632,11 +646,14 @@ extern "C" int ia_group_norm_gate(void* out, const float* o, const float* den, c
     const long long units = (long long)n * (inner / group);
     IA_CHECK(units < 2147483647LL, "group_norm_gate: %d tokens x %d groups exceed the grid", n, inner / group);
     if (group > 256) {
+        // (four features a thread where the group is wide enough: steps of few tokens have few blocks, and a block's
+        // walk over its group is what they wait for)
+        const int threads = group >= 4096 ? 1024 : group >= 2048 ? 512 : 256;
         if (dtype == IA_F32)
-            group_norm_gate_block_kernel<float><<<(unsigned)units, 256, 0, stream>>>((float*)out, o, den, floor_, head, (const float*)gate,
+            group_norm_gate_block_kernel<float><<<(unsigned)units, threads, 0, stream>>>((float*)out, o, den, floor_, head, (const float*)gate,
                                                                                   g_ld, g_off, act, gate_first, w, eps, inner, group);
         else
-            group_norm_gate_block_kernel<bf16_t><<<(unsigned)units, 256, 0, stream>>>((bf16_t*)out, o, den, floor_, head,
+            group_norm_gate_block_kernel<bf16_t><<<(unsigned)units, threads, 0, stream>>>((bf16_t*)out, o, den, floor_, head,
                                                                                    (const bf16_t*)gate, g_ld, g_off, act, gate_first, w,
                                                                                    eps, inner, group);
         IA_LAUNCH_CHECK("group_norm_gate (blocks)");

@@ -8,7 +8,7 @@ output projection.  q head h reads kv head h // (n_heads / n_kv_heads)
 (`attention_utils.rs:38-49`).
 
 Options of the spec beyond the reference's layer: biases, a window, a sink in the softmax (`sink`: the denominator
-holds one more term, exp(0)), values that are the keys as projected, before norm and rotation (`values_from_keys`: no
+holds one more term, exp(0)), values that are the key projection's own rows, ahead of norm and rotation (`values_from_keys`: no
 value projection is loaded; the key projection's rows stand twice in the fused product, so the kernels that take
 [q | k | v] serve unchanged), and other names for the tensors in the file (`names`).
 """

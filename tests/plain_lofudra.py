@@ -50,7 +50,7 @@ def dense_ff(h: torch.Tensor, w: T, p: str) -> torch.Tensor:
     return gelu_erf(h @ w[p + "up"].T) @ w[p + "down"].T
 
 
-# ---- the windowed attention with a sink, values = keys as projected -------------------------------
+# ---- the windowed attention with a sink; its values are its un-normed, un-rotated keys ----------------
 
 def rotate_halves(x: torch.Tensor, positions: torch.Tensor, base: float, dims: int) -> torch.Tensor:
     """x [tokens, heads, dim]: the first `dims` features of every head turn, feature i with i + dims/2."""
@@ -70,7 +70,7 @@ def sink_window_attention(h: torch.Tensor, w: T, p: str, m: dict, eps: float) ->
     window, scale = int((m.get("mask") or {}).get("size", n + 1)), float(m["scale"])      # no mask: every earlier key
     q = (h @ w[p + "q"].T + w[p + "q.b"]).view(n, H, d)
     k = (h @ w[p + "k"].T + w[p + "k.b"]).view(n, G, d)
-    v = k                                             # the values: the keys before norm and rotation
+    v = k                                             # (no value projection: the key rows themselves, ahead of norm and turn)
     pos = torch.arange(n)
     rot = m.get("rot") or {}
     q = rotate_halves(rms_norm(q, w[p + "q.norm"], eps), pos, float(rot.get("base", 1.0)), int(rot.get("dims", 0)))
@@ -141,7 +141,7 @@ def mlstm(h: torch.Tensor, w: T, p: str, m: dict, eps: float) -> torch.Tensor:
 # ---- the selective state space ---------------------------------------------------------------------
 
 def causal_conv(x: torch.Tensor, taps: torch.Tensor, bias: torch.Tensor) -> torch.Tensor:
-    """x [tokens, channels], taps [channels, taps]: the last tap meets the current token, zeros before the start."""
+    """x [tokens, channels], taps [channels, taps]: the last tap meets the current token; ahead of a sequence's first token there is nothing but zeros."""
     n, k = x.shape[0], taps.shape[1]
     padded = torch.cat([torch.zeros(k - 1, x.shape[1], dtype=x.dtype), x], dim=0)
     out = bias.expand(n, -1).clone()
@@ -169,7 +169,7 @@ def mamba2(h: torch.Tensor, w: T, p: str, m: dict, eps: float) -> torch.Tensor:
         for t in range(n):
             S = torch.exp(-rate[head] * dt[t, head]) * S + dt[t, head] * torch.outer(B[t, g], x[t, head])
             y[t, head] = S.T @ C[t, g] + w[p + "D"][head] * x[t, head]
-    y = y.reshape(n, inner) * silu(z)                               # the gate comes before the norm
+    y = y.reshape(n, inner) * silu(z)                               # gated first, normed second
     y = rms_norm(y.view(n, parts, inner // parts), None, eps).reshape(n, inner) * w[p + "norm"]
     return y @ w[p + "o"].T
 
