@@ -223,6 +223,9 @@ int ia_linear_scan(float* out, float* den, float* state, long long row_floats, l
                    float q_scale, float k_scale, int chunk, int max_q_len, float* workspace, int dtype,
                    hipStream_t stream);
 long long ia_linear_scan_workspace(int n_seqs, int max_q_len, int chunk, int H, int dim, int vdim, int normaliser);
+// 1 (the default): what a chunk's start contributes is formed on the matrix cores in true 32-bit (keys up to 128, chunks up
+// to 64 tokens); 0: on the vector units
+void ia_linear_scan_tune(int carry_mfma);
 // [o / (max(|den|, floor) + 1e-6)] [* act(gate)] -> RMS norm in groups of `group` features [* w] [* act(gate)]; act: 1 SiLU, 4 sigmoid
 int ia_group_norm_gate(void* out, const float* o, const float* den, const float* floor_, int head,
                        const void* gate, long long g_ld, int g_off, int act, int gate_first, const float* w,

@@ -442,6 +442,85 @@ __global__ __launch_bounds__(LS_THREADS) void linear_scan_kernel(const ScanArgs 
     if (MODE == LS_LOCAL && blockIdx.x == 0 && threadIdx.x == 0) a.chunk_a[(long long)blockIdx.z * a.H + h] = run;
 }
 
+// CARRY on the matrix cores in their true 32-bit form (`v_mfma_f32_16x16x4_f32`: 32-bit operands, products and sums),
+// for keys of up to 128 entries and chunks of up to 64 tokens: a chunk's share of its start is a product of its queries
+// [tokens x dim] with the matrix it starts from [dim x columns], row t scaled by the product of the decays up to t.  A
+// block of four waves owns a (chunk, head, 32 columns); the queries (scaled) and the columns come into shared memory
+// once, rows `ld` floats apart; wave w owns tokens 16 w .. 16 w + 15.  Lane l supplies A[l % 16][l / 16] and
+// B[l / 16][l % 16] of a step of four k and receives D[4 (l / 16) + r][l % 16].
+typedef float ls_f32x4 __attribute__((ext_vector_type(4)));
+#define LC_TOKENS 64
+#define LC_COLS 32
+#define LC_MAX_DIM 128
+
+template <typename T>
+__global__ __launch_bounds__(256) void linear_carry_mfma_kernel(const ScanArgs a, int ld_s) {
+    extern __shared__ __attribute__((aligned(16))) float lc_shared[];
+    float* const q_s = lc_shared;                          // [LC_TOKENS][ld_s]
+    float* const s_s = q_s + LC_TOKENS * ld_s;             // [LC_COLS][ld_s]
+    float* const run_s = s_s + LC_COLS * ld_s;             // [LC_TOKENS]
+    const int h = blockIdx.y;
+    const int seq = blockIdx.z / a.max_chunks, c = blockIdx.z - seq * a.max_chunks;
+    const int vt = a.vdim + (a.den != nullptr ? 1 : 0);
+    const int j0 = blockIdx.x * LC_COLS;
+    const int first = a.cu_tokens[seq] + c * a.chunk, end = a.cu_tokens[seq + 1];
+    if (first >= end) return;                              // (the whole block)
+    const int nt = end - first < a.chunk ? end - first : a.chunk;
+    const int k4 = (a.dim + 3) / 4 * 4;
+    const T* q = (const T*)a.q + a.q_off + (long long)(h / (a.H / a.q_heads)) * a.dim;
+    for (int e = threadIdx.x; e < LC_TOKENS * k4; e += 256) {
+        const int tt = e / k4, i = e - tt * k4;
+        q_s[tt * ld_s + i] = (tt < nt && i < a.dim) ? ld(q + (long long)(first + tt) * a.q_ld + i) * a.q_scale : 0.f;
+    }
+    const float* start = a.chunk_s + ((long long)blockIdx.z * a.H + h) * vt * a.dim;
+    for (int e = threadIdx.x; e < LC_COLS * k4; e += 256) {
+        const int jj = e / k4, i = e - jj * k4;
+        s_s[jj * ld_s + i] = (j0 + jj < vt && i < a.dim) ? start[(long long)(j0 + jj) * a.dim + i] : 0.f;
+    }
+    if (threadIdx.x < LC_TOKENS) {
+        // the products of the decays up to each token: the first wave's lanes load one decay each and fold them by lane shifts
+        const int tt = threadIdx.x;
+        float run = 1.f;
+        if (tt < nt) {
+            const float an = a.log_a[a.a_per_token ? (long long)(first + tt) * a.H + h : h];
+            run = a.a_per_token ? expf(an) : an;
+        }
+#pragma unroll
+        for (int o = 1; o < LC_TOKENS; o <<= 1) {
+            const float before = __shfl_up(run, o, IA_WAVE);
+            if (tt >= o) run *= before;
+        }
+        run_s[tt] = run;
+    }
+    __syncthreads();
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, kq = lane >> 4;
+    ls_f32x4 acc[LC_COLS / 16];
+#pragma unroll
+    for (int ct = 0; ct < LC_COLS / 16; ++ct) acc[ct] = (ls_f32x4){0.f, 0.f, 0.f, 0.f};
+    const float* qa = q_s + (16 * wave + r16) * ld_s + kq;
+    const float* sb = s_s + r16 * ld_s + kq;
+    for (int k0 = 0; k0 < k4; k0 += 4) {
+        const float av = qa[k0];
+#pragma unroll
+        for (int ct = 0; ct < LC_COLS / 16; ++ct)
+            acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, sb[16 * ct * ld_s + k0], acc[ct], 0, 0, 0);
+    }
+#pragma unroll
+    for (int ct = 0; ct < LC_COLS / 16; ++ct) {
+        const int col = j0 + 16 * ct + r16;
+        if (col >= vt) continue;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int tt = 16 * wave + 4 * kq + r;
+            if (tt >= nt) continue;
+            const long long t = first + tt;
+            float* at = col < a.vdim ? a.out + (t * a.H + h) * a.vdim + col : a.den + t * a.H + h;
+            *at = fmaf(run_s[tt], acc[ct][r], *at);
+        }
+    }
+}
+
 // A request's chunks in order, one thread an entry of the heads' matrices: the workspace's U_c becomes the matrix that
 // chunk c starts from, the state row takes the matrix behind the last chunk.
 __global__ void chunk_states_kernel(float* __restrict__ chunk_s, const float* __restrict__ chunk_a, float* __restrict__ state,
@@ -465,6 +544,10 @@ __global__ void chunk_states_kernel(float* __restrict__ chunk_s, const float* __
     }
     *srow = S;
 }
+
+// (tests switch the matrix cores' form of CARRY off to compare it with the vector units')
+static int g_carry_mfma = 1;
+extern "C" void ia_linear_scan_tune(int carry_mfma) { g_carry_mfma = carry_mfma; }
 
 extern "C" long long ia_linear_scan_workspace(int n_seqs, int max_q_len, int chunk, int H, int dim, int vdim, int normaliser) {
     if (chunk <= 0 || n_seqs <= 0) return 0;
@@ -547,7 +630,15 @@ extern "C" int ia_linear_scan(float* out, float* den, float* state, long long ro
     LS_LAUNCH(LS_LOCAL, grid);
     chunk_states_kernel<<<sgrid, 256, 0, stream>>>(a.chunk_s, a.chunk_a, state, row_floats, s_off, cu_tokens, state_slots, per_head,
                                                    H, chunk, a.max_chunks);
-    LS_LAUNCH(LS_CARRY, grid);
+    if (g_carry_mfma && dim <= LC_MAX_DIM && chunk <= LC_TOKENS) {
+        const int ld_s = (dim + 3) / 4 * 4 + 4;
+        const dim3 cgrid((unsigned)((vt + LC_COLS - 1) / LC_COLS), (unsigned)H, (unsigned)(n_seqs * a.max_chunks));
+        const size_t cshm = (size_t)((LC_TOKENS + LC_COLS) * ld_s + LC_TOKENS) * sizeof(float);
+        if (dtype == IA_F32) linear_carry_mfma_kernel<float><<<cgrid, 256, cshm, stream>>>(a, ld_s);
+        else linear_carry_mfma_kernel<bf16_t><<<cgrid, 256, cshm, stream>>>(a, ld_s);
+    } else {
+        LS_LAUNCH(LS_CARRY, grid);
+    }
 #undef LS_LAUNCH
 #undef LS_LAUNCH_P
     IA_LAUNCH_CHECK("linear_scan (chunks)");

@@ -336,10 +336,16 @@ def test_scan_in_chunks_is_the_walk(H, qh, dim, vdim, normaliser, dtype):
     for gates in (dict(log_a=log_a, b=b), dict(decay=decay)):
         walk = run(0, **gates)
         assert torch.equal(walk[-1][[1, 4]], start[[1, 4]].double()) and torch.equal(walk[-1][:, :7], start[:, :7].double())
-        for chunk in (16, 64, None):
-            for got, want in zip(run(chunk, **gates), walk):
+        for chunk, matrix_cores in ((16, 1), (64, 1), (None, 1), (16, 0), (64, 0)):
+            # (what a chunk's start contributes: on the matrix cores in true 32-bit, or on the vector units)
+            ops.library().ia_linear_scan_tune(matrix_cores)
+            try:
+                results = run(chunk, **gates)
+            finally:
+                ops.library().ia_linear_scan_tune(1)
+            for got, want in zip(results, walk):
                 scale = float(want.abs().max())
-                assert float((got - want).abs().max()) <= 2e-5 * scale, (chunk, float((got - want).abs().max()) / scale)
+                assert float((got - want).abs().max()) <= 2e-5 * scale, (chunk, matrix_cores, float((got - want).abs().max()) / scale)
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
