@@ -521,6 +521,151 @@ __global__ __launch_bounds__(256) void linear_carry_mfma_kernel(const ScanArgs a
     }
 }
 
+// LOCAL on the same instruction, for the same sizes: a block of four waves owns a (chunk, head).  With G_t the sum of
+// the decays' logarithms up to t (inclusive) and b_s the input scales,
+//     P[t][s] = (q_t . k_s) exp(G_t - G_s) b_s  for s <= t (0 beyond),      out_t = sum_s P[t][s] v_s (+ skip v_t),
+//     U = sum_s exp(G_last - G_s) b_s k_s v_s^T,                             A = exp(G_last).
+// The queries and keys of the chunk (scaled, zeros for tokens it does not have) come into shared memory once; the
+// scores are formed once and weighted, then the columns of v come 32 at a time: a product with P for the outputs, a
+// product with the weighted keys for the chunk's matrix.  Every exponent is <= 0.  A decay of 0 has the logarithm
+// -1e4, so that differences stay numbers.  Wave w owns tokens 16 w .. 16 w + 15 of the outputs and rows 16 w .., 16 (w +
+// 4) .. of the chunk's matrix.
+#define LL_P_LD 68
+#define LL_V_LD 36
+
+template <typename T>
+__global__ __launch_bounds__(256) void linear_local_mfma_kernel(const ScanArgs a, int ld_s) {
+    extern __shared__ __attribute__((aligned(16))) float ll_shared[];
+    float* const q_s = ll_shared;                          // [64][ld_s]
+    float* const k_s = q_s + LC_TOKENS * ld_s;             // [64][ld_s]
+    float* const p_s = k_s + LC_TOKENS * ld_s;             // [64][LL_P_LD]
+    float* const v_s = p_s + LC_TOKENS * LL_P_LD;          // [64][LL_V_LD]
+    float* const g_s = v_s + LC_TOKENS * LL_V_LD;          // [64] G_t
+    float* const b_s = g_s + LC_TOKENS;                    // [64] b_s
+    float* const w_s = b_s + LC_TOKENS;                    // [64] exp(G_last - G_s) b_s
+    const int h = blockIdx.y;
+    const int seq = blockIdx.z / a.max_chunks, c = blockIdx.z - seq * a.max_chunks;
+    const int vt = a.vdim + (a.den != nullptr ? 1 : 0);
+    const int first = a.cu_tokens[seq] + c * a.chunk, end = a.cu_tokens[seq + 1];
+    if (first >= end) return;                              // (the whole block)
+    const int nt = end - first < a.chunk ? end - first : a.chunk;
+    const int k4 = (a.dim + 3) / 4 * 4;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int r16 = lane & 15, kq = lane >> 4;
+    const T* q = (const T*)a.q + a.q_off + (long long)(h / (a.H / a.q_heads)) * a.dim;
+    const T* k = (const T*)a.k + a.k_off + (long long)(h / (a.H / a.k_heads)) * a.dim;
+    const T* v = (const T*)a.v + a.v_off + (long long)h * a.vdim;
+    for (int tt = threadIdx.x >> 5; tt < LC_TOKENS; tt += 8)
+        for (int i = threadIdx.x & 31; i < k4; i += 32) {
+            const bool in = tt < nt && i < a.dim;
+            q_s[tt * ld_s + i] = in ? ld(q + (long long)(first + tt) * a.q_ld + i) * a.q_scale : 0.f;
+            k_s[tt * ld_s + i] = in ? ld(k + (long long)(first + tt) * a.k_ld + i) * a.k_scale : 0.f;
+        }
+    if (threadIdx.x < LC_TOKENS) {
+        const int tt = threadIdx.x;
+        float g = 0.f, b = 0.f;
+        if (tt < nt) {
+            const float an = a.log_a[a.a_per_token ? (long long)(first + tt) * a.H + h : h];
+            g = fmaxf(a.a_per_token ? an : logf(an), -1e4f);
+            b = a.b != nullptr ? a.b[(long long)(first + tt) * a.H + h] : 1.f;
+        }
+#pragma unroll
+        for (int o = 1; o < LC_TOKENS; o <<= 1) {
+            const float before = __shfl_up(g, o, IA_WAVE);
+            if (tt >= o) g += before;
+        }
+        const float g_last = __shfl(g, LC_TOKENS - 1, IA_WAVE);
+        g_s[tt] = g; b_s[tt] = b; w_s[tt] = expf(g_last - g) * b;
+        if (tt == 0) a.chunk_a[(long long)blockIdx.z * a.H + h] = expf(g_last);
+    }
+    __syncthreads();
+    // ---- the weighted scores ------------------------------------------------------------------------------------
+    {
+        ls_f32x4 acc[4];
+#pragma unroll
+        for (int ct = 0; ct < 4; ++ct) acc[ct] = (ls_f32x4){0.f, 0.f, 0.f, 0.f};
+        const float* qa = q_s + (16 * wave + r16) * ld_s + kq;
+        const float* kb = k_s + r16 * ld_s + kq;
+        for (int k0 = 0; k0 < k4; k0 += 4) {
+            const float av = qa[k0];
+#pragma unroll
+            for (int ct = 0; ct < 4; ++ct)
+                acc[ct] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, kb[16 * ct * ld_s + k0], acc[ct], 0, 0, 0);
+        }
+#pragma unroll
+        for (int ct = 0; ct < 4; ++ct) {
+            const int s = 16 * ct + r16;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int t = 16 * wave + 4 * kq + r;
+                p_s[t * LL_P_LD + s] = s <= t ? acc[ct][r] * expf(g_s[t] - g_s[s]) * b_s[s] : 0.f;
+            }
+        }
+    }
+    const float skip = a.skip != nullptr ? a.skip[h] : 0.f;
+    float* const u_out = a.chunk_s + ((long long)blockIdx.z * a.H + h) * vt * a.dim;
+    const int row_tiles = (a.dim + 15) / 16;
+    for (int j0 = 0; j0 < vt; j0 += 32) {
+        __syncthreads();                                   // (the scores are written; the columns before are used up)
+        for (int tt = threadIdx.x >> 5; tt < LC_TOKENS; tt += 8) {
+            const int j = j0 + (threadIdx.x & 31);
+            v_s[tt * LL_V_LD + (threadIdx.x & 31)] =
+                (tt < nt && j < vt) ? (j < a.vdim ? ld(v + (long long)(first + tt) * a.v_ld + j) : 1.f) : 0.f;
+        }
+        __syncthreads();
+        // the outputs of the chunk's own tokens
+        {
+            ls_f32x4 acc[2] = {(ls_f32x4){0.f, 0.f, 0.f, 0.f}, (ls_f32x4){0.f, 0.f, 0.f, 0.f}};
+            const float* pa = p_s + (16 * wave + r16) * LL_P_LD + kq;
+            const float* vb = v_s + kq * LL_V_LD + r16;
+#pragma unroll 4
+            for (int k0 = 0; k0 < LC_TOKENS; k0 += 4) {
+                const float av = pa[k0];
+                acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, vb[k0 * LL_V_LD], acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, vb[k0 * LL_V_LD + 16], acc[1], 0, 0, 0);
+            }
+#pragma unroll
+            for (int c2 = 0; c2 < 2; ++c2) {
+                const int col = j0 + 16 * c2 + r16;
+                if (col >= vt) continue;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int tt = 16 * wave + 4 * kq + r;
+                    if (tt >= nt) continue;
+                    const long long t = first + tt;
+                    if (col < a.vdim) a.out[(t * a.H + h) * a.vdim + col] = fmaf(skip, v_s[tt * LL_V_LD + 16 * c2 + r16], acc[c2][r]);
+                    else a.den[t * a.H + h] = acc[c2][r];
+                }
+            }
+        }
+        // the chunk's matrix: rows 16 mt .. of U against these columns
+        for (int mt = wave; mt < row_tiles; mt += 4) {
+            ls_f32x4 acc[2] = {(ls_f32x4){0.f, 0.f, 0.f, 0.f}, (ls_f32x4){0.f, 0.f, 0.f, 0.f}};
+            const float* ka = k_s + kq * ld_s + 16 * mt + r16;
+            const float* vb = v_s + kq * LL_V_LD + r16;
+#pragma unroll 4
+            for (int k0 = 0; k0 < LC_TOKENS; k0 += 4) {
+                const float av = ka[k0 * ld_s] * w_s[k0 + kq];
+                acc[0] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, vb[k0 * LL_V_LD], acc[0], 0, 0, 0);
+                acc[1] = __builtin_amdgcn_mfma_f32_16x16x4f32(av, vb[k0 * LL_V_LD + 16], acc[1], 0, 0, 0);
+            }
+#pragma unroll
+            for (int c2 = 0; c2 < 2; ++c2) {
+                const int col = j0 + 16 * c2 + r16;
+                if (col >= vt) continue;
+                const int i = 16 * mt + 4 * kq;
+                float* at = u_out + (long long)col * a.dim + i;
+                if (a.wide && i + 4 <= a.dim) *(float4*)at = make_float4(acc[c2][0], acc[c2][1], acc[c2][2], acc[c2][3]);
+                else {
+#pragma unroll
+                    for (int r = 0; r < 4; ++r)
+                        if (i + r < a.dim) at[r] = acc[c2][r];
+                }
+            }
+        }
+    }
+}
+
 // A request's chunks in order, one thread an entry of the heads' matrices: the workspace's U_c becomes the matrix that
 // chunk c starts from, the state row takes the matrix behind the last chunk.
 __global__ void chunk_states_kernel(float* __restrict__ chunk_s, const float* __restrict__ chunk_a, float* __restrict__ state,
@@ -627,10 +772,28 @@ extern "C" int ia_linear_scan(float* out, float* den, float* state, long long ro
     const dim3 grid(tiles, (unsigned)H, (unsigned)(n_seqs * a.max_chunks));
     const int per_head = vt * dim;
     const dim3 sgrid((unsigned)(((long long)H * per_head + 255) / 256), (unsigned)n_seqs);
-    LS_LAUNCH(LS_LOCAL, grid);
+    const bool cores = g_carry_mfma && dim <= LC_MAX_DIM && chunk <= LC_TOKENS;
+    if (cores) {
+        const int ld_s = (dim + 3) / 4 * 4 + 4;
+        const dim3 lgrid(1, (unsigned)H, (unsigned)(n_seqs * a.max_chunks));
+        const int lshm = (int)((2 * LC_TOKENS * ld_s + LC_TOKENS * (LL_P_LD + LL_V_LD) + 3 * LC_TOKENS) * sizeof(float));
+        static int asked_f32 = 0, asked_bf16 = 0;          // shared memory beyond 64 KiB has to be asked for, once per instantiation
+        int& asked = dtype == IA_F32 ? asked_f32 : asked_bf16;
+        if (lshm > asked) {
+            const hipError_t e = dtype == IA_F32
+                ? hipFuncSetAttribute((const void*)linear_local_mfma_kernel<float>, hipFuncAttributeMaxDynamicSharedMemorySize, 112 * 1024)
+                : hipFuncSetAttribute((const void*)linear_local_mfma_kernel<bf16_t>, hipFuncAttributeMaxDynamicSharedMemorySize, 112 * 1024);
+            IA_CHECK(e == hipSuccess, "linear_scan: cannot ask for %d bytes of shared memory: %s", 112 * 1024, hipGetErrorString(e));
+            asked = 112 * 1024;
+        }
+        if (dtype == IA_F32) linear_local_mfma_kernel<float><<<lgrid, 256, lshm, stream>>>(a, ld_s);
+        else linear_local_mfma_kernel<bf16_t><<<lgrid, 256, lshm, stream>>>(a, ld_s);
+    } else {
+        LS_LAUNCH(LS_LOCAL, grid);
+    }
     chunk_states_kernel<<<sgrid, 256, 0, stream>>>(a.chunk_s, a.chunk_a, state, row_floats, s_off, cu_tokens, state_slots, per_head,
                                                    H, chunk, a.max_chunks);
-    if (g_carry_mfma && dim <= LC_MAX_DIM && chunk <= LC_TOKENS) {
+    if (cores) {
         const int ld_s = (dim + 3) / 4 * 4 + 4;
         const dim3 cgrid((unsigned)((vt + LC_COLS - 1) / LC_COLS), (unsigned)H, (unsigned)(n_seqs * a.max_chunks));
         const size_t cshm = (size_t)((LC_TOKENS + LC_COLS) * ld_s + LC_TOKENS) * sizeof(float);
