@@ -330,6 +330,7 @@ struct ScanArgs {
     int H, dim, vdim, P, cols;                                    // cols: columns of S a block (LS_THREADS / P)
     float q_scale, k_scale;
     int wide;                                                     // the matrices' rows start at multiples of 16 bytes
+    int q_vec, k_vec;                                             // so do the heads' rows of q and k, and dim is a multiple of a 16-byte load
     int stage;                                                    // tokens whose operands a block holds in shared memory at a time
     int chunk, max_chunks;                                        // LOCAL, CARRY: tokens of a chunk; chunks of the longest portion
     float* chunk_s;                                               // [seqs][max_chunks][H][vt][dim]
@@ -450,6 +451,63 @@ __global__ __launch_bounds__(LS_THREADS) void linear_scan_kernel(const ScanArgs 
 // B[l / 16][l % 16] of a step of four k and receives D[4 (l / 16) + r][l % 16].
 typedef float ls_f32x4 __attribute__((ext_vector_type(4)));
 #define LC_TOKENS 64
+
+// Rows of a chunk into shared memory as 32-bit values times `scale`: dst[tt][i] = src[(first + tt) * src_ld + i] for tt <
+// nt and i < dim, zeros up to 64 rows and k4 columns.  `vec`: 16-byte loads (the rows start at multiples of 16 bytes and
+// dim is a multiple of what a load holds); every load of a thread is asked for before its first store.
+__device__ __forceinline__ void ls_load16(const float* p, float (&v)[8], int& n) {
+    const float4 q = *(const float4*)p;
+    v[0] = q.x; v[1] = q.y; v[2] = q.z; v[3] = q.w; n = 4;
+}
+__device__ __forceinline__ void ls_load16(const bf16_t* p, float (&v)[8], int& n) { ls_unpack8(p, v); n = 8; }
+
+template <typename T>
+__device__ __forceinline__ void stage_rows(float* __restrict__ dst, int ld_s, const T* __restrict__ src, long long src_ld,
+                                           int first, int nt, int dim, int k4, float scale, bool vec) {
+    constexpr int E = 16 / (int)sizeof(T);                // elements a load
+    if (vec) {
+        const int per_row = dim / E;                       // (k4 == dim here)
+        const int total = LC_TOKENS * per_row;             // at most 64 * 32 = 8 rounds of the block
+        float v[8][8];
+        int n = E;
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            const int idx = threadIdx.x + 256 * it;
+            const int tt = idx / per_row, piece = idx - tt * per_row;
+            if (idx < total && tt < nt) ls_load16(src + (long long)(first + tt) * src_ld + piece * E, v[it], n);
+            else {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) v[it][e] = 0.f;
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < 8; ++it) {
+            const int idx = threadIdx.x + 256 * it;
+            const int tt = idx / per_row, piece = idx - tt * per_row;
+            if (idx < total) {
+#pragma unroll
+                for (int e = 0; e < E; ++e) dst[tt * ld_s + piece * E + e] = v[it][e] * scale;
+            }
+        }
+        return;
+    }
+    // element by element: 8 rows x 4 columns a thread (k4 <= 128), the loads first
+    float v[8][4];
+#pragma unroll
+    for (int it = 0; it < 8; ++it)
+#pragma unroll
+        for (int ic = 0; ic < 4; ++ic) {
+            const int tt = (threadIdx.x >> 5) + 8 * it, i = (threadIdx.x & 31) + 32 * ic;
+            v[it][ic] = (tt < nt && i < dim) ? ld(src + (long long)(first + tt) * src_ld + i) : 0.f;
+        }
+#pragma unroll
+    for (int it = 0; it < 8; ++it)
+#pragma unroll
+        for (int ic = 0; ic < 4; ++ic) {
+            const int tt = (threadIdx.x >> 5) + 8 * it, i = (threadIdx.x & 31) + 32 * ic;
+            if (i < k4) dst[tt * ld_s + i] = v[it][ic] * scale;
+        }
+}
 #define LC_COLS 32
 #define LC_MAX_DIM 128
 
@@ -468,14 +526,22 @@ __global__ __launch_bounds__(256) void linear_carry_mfma_kernel(const ScanArgs a
     const int nt = end - first < a.chunk ? end - first : a.chunk;
     const int k4 = (a.dim + 3) / 4 * 4;
     const T* q = (const T*)a.q + a.q_off + (long long)(h / (a.H / a.q_heads)) * a.dim;
-    for (int e = threadIdx.x; e < LC_TOKENS * k4; e += 256) {
-        const int tt = e / k4, i = e - tt * k4;
-        q_s[tt * ld_s + i] = (tt < nt && i < a.dim) ? ld(q + (long long)(first + tt) * a.q_ld + i) * a.q_scale : 0.f;
-    }
+    stage_rows<T>(q_s, ld_s, q, a.q_ld, first, nt, a.dim, k4, a.q_scale, a.q_vec != 0);
+    // (the columns of the start's matrix lie like rows of dim entries: the same staging, 32 of them)
     const float* start = a.chunk_s + ((long long)blockIdx.z * a.H + h) * vt * a.dim;
-    for (int e = threadIdx.x; e < LC_COLS * k4; e += 256) {
-        const int jj = e / k4, i = e - jj * k4;
-        s_s[jj * ld_s + i] = (j0 + jj < vt && i < a.dim) ? start[(long long)(j0 + jj) * a.dim + i] : 0.f;
+    const int cols_here = vt - j0 < LC_COLS ? vt - j0 : LC_COLS;
+    if (a.wide) {
+        const int per_row = a.dim / 4;
+        for (int idx = threadIdx.x; idx < LC_COLS * per_row; idx += 256) {
+            const int jj = idx / per_row, piece = idx - jj * per_row;
+            const float4 z = jj < cols_here ? *(const float4*)(start + (long long)(j0 + jj) * a.dim + 4 * piece) : make_float4(0.f, 0.f, 0.f, 0.f);
+            *(float4*)(s_s + jj * ld_s + 4 * piece) = z;
+        }
+    } else {
+        for (int e = threadIdx.x; e < LC_COLS * k4; e += 256) {
+            const int jj = e / k4, i = e - jj * k4;
+            s_s[jj * ld_s + i] = (jj < cols_here && i < a.dim) ? start[(long long)(j0 + jj) * a.dim + i] : 0.f;
+        }
     }
     if (threadIdx.x < LC_TOKENS) {
         // the products of the decays up to each token: the first wave's lanes load one decay each and fold them by lane shifts
@@ -555,12 +621,8 @@ __global__ __launch_bounds__(256) void linear_local_mfma_kernel(const ScanArgs a
     const T* q = (const T*)a.q + a.q_off + (long long)(h / (a.H / a.q_heads)) * a.dim;
     const T* k = (const T*)a.k + a.k_off + (long long)(h / (a.H / a.k_heads)) * a.dim;
     const T* v = (const T*)a.v + a.v_off + (long long)h * a.vdim;
-    for (int tt = threadIdx.x >> 5; tt < LC_TOKENS; tt += 8)
-        for (int i = threadIdx.x & 31; i < k4; i += 32) {
-            const bool in = tt < nt && i < a.dim;
-            q_s[tt * ld_s + i] = in ? ld(q + (long long)(first + tt) * a.q_ld + i) * a.q_scale : 0.f;
-            k_s[tt * ld_s + i] = in ? ld(k + (long long)(first + tt) * a.k_ld + i) * a.k_scale : 0.f;
-        }
+    stage_rows<T>(q_s, ld_s, q, a.q_ld, first, nt, a.dim, k4, a.q_scale, a.q_vec != 0);
+    stage_rows<T>(k_s, ld_s, k, a.k_ld, first, nt, a.dim, k4, a.k_scale, a.k_vec != 0);
     if (threadIdx.x < LC_TOKENS) {
         const int tt = threadIdx.x;
         float g = 0.f, b = 0.f;
@@ -607,10 +669,16 @@ __global__ __launch_bounds__(256) void linear_local_mfma_kernel(const ScanArgs a
     const int row_tiles = (a.dim + 15) / 16;
     for (int j0 = 0; j0 < vt; j0 += 32) {
         __syncthreads();                                   // (the scores are written; the columns before are used up)
-        for (int tt = threadIdx.x >> 5; tt < LC_TOKENS; tt += 8) {
+        {
             const int j = j0 + (threadIdx.x & 31);
-            v_s[tt * LL_V_LD + (threadIdx.x & 31)] =
-                (tt < nt && j < vt) ? (j < a.vdim ? ld(v + (long long)(first + tt) * a.v_ld + j) : 1.f) : 0.f;
+            float vv[8];
+#pragma unroll
+            for (int it = 0; it < 8; ++it) {
+                const int tt = (threadIdx.x >> 5) + 8 * it;
+                vv[it] = (tt < nt && j < vt) ? (j < a.vdim ? ld(v + (long long)(first + tt) * a.v_ld + j) : 1.f) : 0.f;
+            }
+#pragma unroll
+            for (int it = 0; it < 8; ++it) v_s[((threadIdx.x >> 5) + 8 * it) * LL_V_LD + (threadIdx.x & 31)] = vv[it];
         }
         __syncthreads();
         // the outputs of the chunk's own tokens
@@ -735,6 +803,11 @@ extern "C" int ia_linear_scan(float* out, float* den, float* state, long long ro
     a.q_scale = q_scale; a.k_scale = k_scale;
     a.chunk = chunk; a.max_chunks = chunk ? (max_q_len + chunk - 1) / chunk : 1;
     a.chunk_s = workspace;
+    {
+        const int per = dtype == IA_F32 ? 4 : 8;                  // elements a 16-byte load
+        a.q_vec = dim % per == 0 && q_off % per == 0 && q_ld % per == 0 && ((uintptr_t)q & 15) == 0;
+        a.k_vec = dim % per == 0 && k_off % per == 0 && k_ld % per == 0 && ((uintptr_t)k & 15) == 0;
+    }
     a.wide = dim % 4 == 0 && s_off % 4 == 0 && row_floats % 4 == 0 && ((uintptr_t)state & 15) == 0 && ((uintptr_t)workspace & 15) == 0;
     a.chunk_a = workspace ? workspace + (long long)n_seqs * a.max_chunks * H * vt * dim : nullptr;
     IA_CHECK((long long)n_seqs * a.max_chunks <= 65535, "linear_scan: %d requests x %d chunks exceed the grid", n_seqs, a.max_chunks);
