@@ -304,7 +304,8 @@ def test_convolution_with_its_tail(C, ld, off, taps, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("H,qh,dim,vdim,normaliser", [(3, 3, 10, 12, False), (4, 2, 24, 9, True), (2, 1, 128, 64, True), (8, 8, 64, 128, False)])
+@pytest.mark.parametrize("H,qh,dim,vdim,normaliser", [(3, 3, 10, 12, False), (4, 2, 24, 9, True), (2, 1, 128, 64, True), (8, 8, 64, 128, False),
+                                                      (2, 2, 256, 16, True), (1, 1, 512, 8, False), (2, 1, 132, 40, False)])
 def test_scan_in_chunks_is_the_walk(H, qh, dim, vdim, normaliser, dtype):
     """Three requests of unequal lengths in one step, from states that are not zero: chunks of 16 and of 64 tokens side
     by side give what the walk token by token gives, outputs and final states, up to rounding; so do decays that are
@@ -336,7 +337,7 @@ def test_scan_in_chunks_is_the_walk(H, qh, dim, vdim, normaliser, dtype):
     for gates in (dict(log_a=log_a, b=b), dict(decay=decay)):
         walk = run(0, **gates)
         assert torch.equal(walk[-1][[1, 4]], start[[1, 4]].double()) and torch.equal(walk[-1][:, :7], start[:, :7].double())
-        for chunk, matrix_cores in ((16, 1), (64, 1), (None, 1), (16, 0), (64, 0)):
+        for chunk, matrix_cores in ((16, 1), (64, 1), (None, 1), (16, 0), (64, 0), (128, 1)):
             # (what a chunk's start contributes: on the matrix cores in true 32-bit, or on the vector units)
             ops.library().ia_linear_scan_tune(matrix_cores)
             try:
