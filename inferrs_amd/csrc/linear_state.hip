@@ -602,10 +602,15 @@ __global__ __launch_bounds__(256) void linear_carry_mfma_kernel(const ScanArgs a
 template <typename T>
 __global__ __launch_bounds__(256) void linear_local_mfma_kernel(const ScanArgs a, int ld_s) {
     extern __shared__ __attribute__((aligned(16))) float ll_shared[];
+    // (The scores take the place of the queries where a row of queries is long enough for a row of scores: a wave
+    // writes the scores of its 16 tokens after it has read those tokens' queries, and nobody else reads them.  Two
+    // blocks then fit a compute unit's shared memory at keys of 128.)
+    const bool over = ld_s >= LL_P_LD;
+    const int p_ld = over ? ld_s : LL_P_LD;
     float* const q_s = ll_shared;                          // [64][ld_s]
     float* const k_s = q_s + LC_TOKENS * ld_s;             // [64][ld_s]
-    float* const p_s = k_s + LC_TOKENS * ld_s;             // [64][LL_P_LD]
-    float* const v_s = p_s + LC_TOKENS * LL_P_LD;          // [64][LL_V_LD]
+    float* const p_s = over ? q_s : k_s + LC_TOKENS * ld_s;   // [64][p_ld]
+    float* const v_s = k_s + LC_TOKENS * ld_s + (over ? 0 : LC_TOKENS * LL_P_LD);   // [64][LL_V_LD]
     float* const g_s = v_s + LC_TOKENS * LL_V_LD;          // [64] G_t
     float* const b_s = g_s + LC_TOKENS;                    // [64] b_s
     float* const w_s = b_s + LC_TOKENS;                    // [64] exp(G_last - G_s) b_s
@@ -660,7 +665,7 @@ __global__ __launch_bounds__(256) void linear_local_mfma_kernel(const ScanArgs a
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int t = 16 * wave + 4 * kq + r;
-                p_s[t * LL_P_LD + s] = s <= t ? acc[ct][r] * expf(g_s[t] - g_s[s]) * b_s[s] : 0.f;
+                p_s[t * p_ld + s] = s <= t ? acc[ct][r] * expf(g_s[t] - g_s[s]) * b_s[s] : 0.f;
             }
         }
     }
@@ -684,7 +689,7 @@ __global__ __launch_bounds__(256) void linear_local_mfma_kernel(const ScanArgs a
         // the outputs of the chunk's own tokens
         {
             ls_f32x4 acc[2] = {(ls_f32x4){0.f, 0.f, 0.f, 0.f}, (ls_f32x4){0.f, 0.f, 0.f, 0.f}};
-            const float* pa = p_s + (16 * wave + r16) * LL_P_LD + kq;
+            const float* pa = p_s + (16 * wave + r16) * p_ld + kq;
             const float* vb = v_s + kq * LL_V_LD + r16;
 #pragma unroll 4
             for (int k0 = 0; k0 < LC_TOKENS; k0 += 4) {
@@ -849,7 +854,7 @@ extern "C" int ia_linear_scan(float* out, float* den, float* state, long long ro
     if (cores) {
         const int ld_s = (dim + 3) / 4 * 4 + 4;
         const dim3 lgrid(1, (unsigned)H, (unsigned)(n_seqs * a.max_chunks));
-        const int lshm = (int)((2 * LC_TOKENS * ld_s + LC_TOKENS * (LL_P_LD + LL_V_LD) + 3 * LC_TOKENS) * sizeof(float));
+        const int lshm = (int)((2 * LC_TOKENS * ld_s + LC_TOKENS * ((ld_s >= LL_P_LD ? 0 : LL_P_LD) + LL_V_LD) + 3 * LC_TOKENS) * sizeof(float));
         static int asked_f32 = 0, asked_bf16 = 0;          // shared memory beyond 64 KiB has to be asked for, once per instantiation
         int& asked = dtype == IA_F32 ? asked_f32 : asked_bf16;
         if (lshm > asked) {
