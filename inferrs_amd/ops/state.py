@@ -146,8 +146,9 @@ def linear_scan(*, q: torch.Tensor, q_off: int, q_heads: int, k: torch.Tensor, k
     one more column whose value is always 1; returns (o, that column's output [n, heads]).  o is 32-bit [n, heads * vdim].
     `max_q_len`: an upper bound of the tokens a request brings (0: unknown, the step's tokens).  `chunk`: 0 walks every
     request's tokens in order; a number cuts portions into chunks of that many tokens that run side by side (three
-    kernels: each chunk from nothing, the chunks' matrices in order, what each chunk's start contributes), which differs
-    from the walk by rounding; None: chunks of `SCAN_CHUNK` for steps with a portion of more than `SCAN_CHUNKS_FROM` tokens."""
+    kernels: each chunk from nothing, the chunks' matrices in order, what each chunk's start contributes; for keys of
+    up to 128 entries and chunks of up to 64 tokens the first and the third are products on the matrix cores in true
+    32-bit), which differs from the walk by rounding; None: chunks of `SCAN_CHUNK` for steps with a portion of more than `SCAN_CHUNKS_FROM` tokens."""
     _dev(q, k, v, state, cu_tokens, state_slots, log_a, decay, b, skip)
     _f32(log_a, "log_a"); _f32(decay, "decay"); _f32(b, "b"); _f32(skip, "skip")
     _i32(cu_tokens, "cu_tokens"); _i32(state_slots, "state_slots")
