@@ -25,7 +25,7 @@ from dataclasses import dataclass
 from typing import Any, Dict, Tuple
 
 from .base import ConfigError
-from .buketar import _get, _int, _num
+from .buketar import _int, _num
 from .spec import (AttentionSpec, DenseMlpSpec, LayerSpec, MatrixMemorySpec, ModelSpec, NormSpec, PassInputSpec,
                    PositionSpec, RetentionSpec, ScheduleEntry, SideBySideSpec, StateSpaceSpec)
 

@@ -14,7 +14,6 @@ A request keeps its matrices (and the running maxima, or the convolution's last 
 """
 from __future__ import annotations
 
-import math
 from typing import Dict
 
 import torch
