@@ -516,6 +516,33 @@ def test_random_weights_engine_steps():
     assert logits.shape == (2, 211) and bool(torch.isfinite(logits).all())
 
 
+def test_command_line_run_and_bench(models):
+    """The command line serves the design as it serves the others: greedy tokens are the plain implementation's, a drawn run
+    and the timing command finish."""
+    import json
+    folder, cfg, tensors, reqs, ref = models[("A", 1.0)]
+    prompt = random_tokens(9, cfg["vocab"], 3)
+    toks = list(prompt)
+    for _ in range(6):
+        toks.append(int(pl.forward(cfg, tensors, toks)[-1].argmax()))
+    exe = [sys.executable, os.path.join(ROOT, "bin", "inferrs-amd")]
+    common = ["--block-size", "16", "--max-blocks", "32", "--max-batch-size", "2"]
+    proc = subprocess.run(exe + ["run", folder, ",".join(map(str, prompt)), "--dtype", "f32", "--temperature", "0",
+                                 "--repetition-penalty", "1.0", "--max-tokens", "6"] + common, capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [int(t) for t in proc.stdout.split()] == toks[len(prompt):]
+    proc = subprocess.run(exe + ["run", folder, ",".join(map(str, prompt)), "--dtype", "bf16", "--seed", "5", "--max-tokens", "12",
+                                 "--ignore-eos"] + common, capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    drawn = [int(t) for t in proc.stdout.split()]
+    assert len(drawn) == 12 and all(0 <= t < cfg["vocab"] for t in drawn)
+    proc = subprocess.run(exe + ["bench", folder, "--dtype", "bf16", "--prompt-len", "40", "--max-tokens", "8", "--runs", "2"] + common,
+                          capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    rec = json.loads(proc.stdout.strip().splitlines()[-1])
+    assert rec["prefill_tok_s"] > 0 and rec["decode_tok_s"] > 0
+
+
 def test_trace_runner_program(models, tmp_path):
     folder, cfg, tensors, reqs, ref = models[("B", 1.0)]
     some = {r: reqs[r] for r in ("r2", "r3", "r4")}
